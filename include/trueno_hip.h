@@ -1,0 +1,149 @@
+/* trueno_hip.h - C ABI of libtrueno_hip.so: the MI355X (gfx950) backend for trueno-gpu's fused
+ * k-quant matrix path.
+ *
+ * What binds here.  trueno-gpu reaches its GPU through a table of 25 `cu*` function pointers
+ * (trueno-gpu/src/driver/sys.rs:99-201) loaded from libcuda (sys.rs:230-257).  Sections 1-6 below
+ * are a one-to-one image of that table over the HIP runtime, so `driver/sys.rs` can bind this
+ * library instead and `driver/{context,module,stream,memory}.rs` stay as they are.  Section 7
+ * replaces "emit PTX, JIT it" (kernels/mod.rs:56-67 + driver/module.rs:62-79) by a code object that
+ * ships inside the library.  Section 8 are typed launchers for the kernels of
+ * trueno-gpu/src/kernels/quantize.rs; they own the launch geometry.  Sections 9-10 have no
+ * counterpart in the reference (timing and a test surface).
+ *
+ * Conventions.  Every call returns a status: 0 = success, otherwise the hipError_t value (the
+ * reference maps any non-zero CUresult to GpuError::CudaDriver(name, code), sys.rs:360-369; a missing
+ * device is hipErrorNoDevice = 100, which maps to GpuError::CudaNotAvailable).  Device pointers
+ * are plain 64-bit integers (CUdeviceptr, sys.rs:60).  The library never owns host memory and never
+ * keeps a host pointer after a synchronous call returns.  Nothing here allocates device memory
+ * except trn_mem_alloc.  All entry points may be called from any thread; calls that touch a device
+ * act on the calling thread's current device (trn_ctx_set_current).
+ */
+#ifndef TRUENO_HIP_H
+#define TRUENO_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRN_API __attribute__((visibility("default")))
+
+typedef int trn_status;                 /* CUresult,    sys.rs:27  */
+typedef int trn_device;                 /* CUdevice,    sys.rs:33  */
+typedef struct trn_ctx_s* trn_ctx;      /* CUcontext,   sys.rs:39  */
+typedef struct trn_module_s* trn_module;     /* CUmodule,    sys.rs:45 */
+typedef struct trn_function_s* trn_function; /* CUfunction,  sys.rs:51 */
+typedef void* trn_stream;               /* CUstream,    sys.rs:57 (NULL = default stream) */
+typedef uint64_t trn_dptr;              /* CUdeviceptr, sys.rs:60 */
+typedef struct trn_event_s* trn_event;
+
+#define TRN_SUCCESS 0
+#define TRN_ERROR_INVALID_VALUE 1       /* hipErrorInvalidValue */
+#define TRN_ERROR_NO_DEVICE 100         /* hipErrorNoDevice */
+#define TRN_ERROR_INVALID_DEVICE 101    /* hipErrorInvalidDevice */
+#define TRN_ERROR_NOT_FOUND 500         /* hipErrorNotFound */
+#define TRN_STREAM_NON_BLOCKING 1u      /* CU_STREAM_NON_BLOCKING, driver/stream.rs:60 */
+
+/* ---- 1. initialisation (sys.rs:101-102) ------------------------------------------------ */
+TRN_API trn_status trn_init(unsigned flags);                                    /* cuInit */
+
+/* ---- 2. devices (sys.rs:104-114) --------------------------------------------------------- */
+TRN_API trn_status trn_device_get_count(int* count);                            /* cuDeviceGetCount */
+TRN_API trn_status trn_device_get(trn_device* device, int ordinal);             /* cuDeviceGet */
+TRN_API trn_status trn_device_get_name(char* name, int len, trn_device device); /* cuDeviceGetName */
+TRN_API trn_status trn_device_total_mem(size_t* bytes, trn_device device);      /* cuDeviceTotalMem_v2 */
+
+/* ---- 3. primary context (sys.rs:116-126) -------------------------------------------------- */
+TRN_API trn_status trn_primary_ctx_retain(trn_ctx* ctx, trn_device device);     /* cuDevicePrimaryCtxRetain */
+TRN_API trn_status trn_primary_ctx_release(trn_device device);                  /* cuDevicePrimaryCtxRelease */
+TRN_API trn_status trn_ctx_set_current(trn_ctx ctx);                            /* cuCtxSetCurrent */
+TRN_API trn_status trn_ctx_synchronize(void);                                   /* cuCtxSynchronize */
+
+/* ---- 4. modules (sys.rs:128-140) ----------------------------------------------------------- */
+/* image: a gfx950 code object (ELF) in host memory, where the reference passes PTX text. */
+TRN_API trn_status trn_module_load_data(trn_module* module, const void* image); /* cuModuleLoadData */
+TRN_API trn_status trn_module_unload(trn_module module);                        /* cuModuleUnload */
+TRN_API trn_status trn_module_get_function(trn_function* func, trn_module module,
+                                           const char* name);                   /* cuModuleGetFunction */
+
+/* ---- 5. memory (sys.rs:142-176) ------------------------------------------------------------ */
+TRN_API trn_status trn_mem_alloc(trn_dptr* ptr, size_t size);                   /* cuMemAlloc_v2 */
+TRN_API trn_status trn_mem_free(trn_dptr ptr);                                  /* cuMemFree_v2; 0 is a no-op */
+TRN_API trn_status trn_memcpy_htod(trn_dptr dst, const void* src, size_t size); /* cuMemcpyHtoD_v2 */
+TRN_API trn_status trn_memcpy_dtoh(void* dst, trn_dptr src, size_t size);       /* cuMemcpyDtoH_v2 */
+TRN_API trn_status trn_memcpy_htod_async(trn_dptr dst, const void* src, size_t size, trn_stream stream); /* cuMemcpyHtoDAsync_v2 */
+TRN_API trn_status trn_memcpy_dtoh_async(void* dst, trn_dptr src, size_t size, trn_stream stream);       /* cuMemcpyDtoHAsync_v2 */
+TRN_API trn_status trn_memcpy_dtod(trn_dptr dst, trn_dptr src, size_t size);    /* cuMemcpyDtoD_v2 */
+TRN_API trn_status trn_memcpy_dtod_async(trn_dptr dst, trn_dptr src, size_t size, trn_stream stream);    /* cuMemcpyDtoDAsync_v2 */
+TRN_API trn_status trn_mem_get_info(size_t* free_bytes, size_t* total_bytes);   /* cuMemGetInfo_v2 */
+
+/* ---- 6. streams and launch (sys.rs:178-200) -------------------------------------------------- */
+TRN_API trn_status trn_stream_create(trn_stream* stream, unsigned flags);       /* cuStreamCreate */
+TRN_API trn_status trn_stream_destroy(trn_stream stream);                       /* cuStreamDestroy_v2 */
+TRN_API trn_status trn_stream_synchronize(trn_stream stream);                   /* cuStreamSynchronize */
+/* cuLaunchKernel.  kernel_params[i] points at a host copy of parameter i, in declared order
+ * (driver/stream.rs:110-154).  For the k-quant kernels of the built-in module the grid, block and
+ * shared-memory arguments are ignored and replaced by the kernel's own geometry (the reference's
+ * documented grid = N blocks of 32 threads, quantize.rs:1151-1155, is a warp32 shape); the result
+ * never depends on the geometry the caller passed.  Other functions launch exactly as given. */
+TRN_API trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y, unsigned grid_z,
+                                     unsigned block_x, unsigned block_y, unsigned block_z,
+                                     unsigned shared_mem_bytes, trn_stream stream,
+                                     void** kernel_params, void** extra);
+
+/* ---- 7. the built-in code object ------------------------------------------------------------- */
+/* Loads the gfx950 code object embedded in this library on the current device.  Stands where the
+ * reference does CudaModule::from_ptx(&ctx, &kernel.emit_ptx()) (driver/module.rs:62-79,
+ * kernels/mod.rs:65-67).  It exports, with the reference's parameter lists:
+ *   q4k_gemv_warp_reduce  q5k_gemv_warp_reduce  q6k_gemv_warp_reduce   (y, w, x, k_dim, n_dim)
+ *   q4k_gemm_ggml         q5k_gemm_ggml         q6k_gemm_ggml          (a, b_quant, c, m, n, k) */
+TRN_API trn_status trn_module_load_builtin(trn_module* module);
+/* Pointer to and size of that embedded code object (for callers that want trn_module_load_data). */
+TRN_API trn_status trn_builtin_image(const void** image, size_t* size);
+
+/* ---- 8. typed launchers ------------------------------------------------------------------------
+ * y[n] = sum_k dequant(W)[n,k] * x[k].  W: n rows x (k/256) super-blocks, row-major, 144/176/210
+ * bytes per super-block; x: k f32; y: n f32.  k must be a multiple of 256 (else
+ * TRN_ERROR_INVALID_VALUE); n = 0 is a no-op; k = 0 writes zeros.  Asynchronous on `stream`.
+ * Replace Q4KGemvKernel / Q5KGemvKernel / Q6KGemvKernel + launch_kernel
+ * (quantize.rs:1156-1523, :1532-1724, :1733-1965). */
+TRN_API trn_status trn_q4k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_dptr x, uint32_t k, uint32_t n);
+TRN_API trn_status trn_q5k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_dptr x, uint32_t k, uint32_t n);
+TRN_API trn_status trn_q6k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_dptr x, uint32_t k, uint32_t n);
+/* C[m x n] = A[m x k] . dequant(W[n x k])^T, c[row*n + col]; A, C f32 row-major.  The decode is the
+ * GEMV-family one, so m = 1 equals the GEMV.  Replace QuantizeKernel::ggml / Q5KKernel / Q6KKernel
+ * (quantize.rs:347-579, :640-866, :926-1121). */
+TRN_API trn_status trn_q4k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+TRN_API trn_status trn_q5k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+
+/* ---- 9. test surface: dequantise to f32 (no counterpart in the reference) ------------------------
+ * out[sb*256 + i] = weight i of super-block sb.  policy 0 = GEMV-family decode
+ * (quantize.rs:1237-1483, :1589-1693, :1806-1934); policy 1 = GEMM-family decode as written
+ * (quantize.rs:445-514, :727-807, :1009-1064). */
+TRN_API trn_status trn_q4k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
+TRN_API trn_status trn_q5k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
+TRN_API trn_status trn_q6k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
+
+/* ---- 10. timing, errors, tuning (no counterpart in the reference) --------------------------------- */
+TRN_API trn_status trn_event_create(trn_event* event);
+TRN_API trn_status trn_event_destroy(trn_event event);
+TRN_API trn_status trn_event_record(trn_event event, trn_stream stream);
+TRN_API trn_status trn_event_synchronize(trn_event event);
+TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop);
+/* dst[0..bytes) = src[0..bytes) with one 16-byte load and store per lane; bytes % 16 == 0.
+ * The plain-copy yardstick that HBM counters are scaled by. */
+TRN_API trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t bytes);
+TRN_API const char* trn_error_name(trn_status status);
+TRN_API const char* trn_error_string(trn_status status);
+/* Number of compute units of the current device (sizes the launches). */
+TRN_API trn_status trn_device_cu_count(int* count);
+/* Launch tuning knobs, process-wide: "gemv_blocks_per_cu", "gemv_row_groups".  0 restores the default. */
+TRN_API trn_status trn_set_tuning(const char* key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRUENO_HIP_H */

@@ -1,0 +1,58 @@
+"""Shared helpers for the GPU parity tests: upload, launch through the C ABI, download."""
+from __future__ import annotations
+
+import numpy as np
+
+import trueno_amd as t
+from trueno_amd import kernels as K
+
+GEMV_KERNEL = {"q4k": t.Q4KGemvKernel, "q5k": t.Q5KGemvKernel, "q6k": t.Q6KGemvKernel}
+GEMM_KERNEL = {"q4k": t.QuantizeKernel.ggml, "q5k": t.Q5KKernel, "q6k": t.Q6KKernel}
+SB = {"q4k": 144, "q5k": 176, "q6k": 210}
+
+
+def gpu_dequant(gpu, fmt: str, buf: np.ndarray, policy: int = 0, w_offset: int = 0) -> np.ndarray:
+    ctx, stream = gpu
+    buf = np.ascontiguousarray(buf, np.uint8).reshape(-1)
+    n_sb = buf.size // SB[fmt]
+    dw = t.GpuBuffer(ctx, buf.size + w_offset, np.uint8)
+    dw.copy_from_host_at(buf, w_offset)
+    out = t.GpuBuffer(ctx, n_sb * 256, np.float32)
+    K.dequant_f32(fmt, stream, out, dw.as_ptr() + w_offset, n_sb, policy)
+    stream.synchronize()
+    return out.copy_to_host().reshape(n_sb, 256)
+
+
+def gpu_gemv(gpu, fmt: str, buf: np.ndarray, x: np.ndarray, k: int, n: int, *, by_name=None,
+             w_offset: int = 0, x_offset: int = 0, fill: float = np.nan) -> np.ndarray:
+    """y = W x on the GPU.  by_name: a CudaModule to go through launch_kernel with the reference's
+    LaunchConfig instead of the typed launcher.  Offsets (bytes / elements) misalign the operands."""
+    ctx, stream = gpu
+    buf = np.ascontiguousarray(buf, np.uint8).reshape(-1)
+    dw = t.GpuBuffer(ctx, buf.size + w_offset, np.uint8)
+    dw.copy_from_host_at(buf, w_offset)
+    dx = t.GpuBuffer(ctx, k + x_offset, np.float32)
+    dx.copy_from_host_at(np.ascontiguousarray(x, np.float32), x_offset)
+    dy = t.GpuBuffer.from_host(ctx, np.full(max(n, 1), fill, np.float32))
+    kern = GEMV_KERNEL[fmt](k, n)
+    wp, xp = dw.as_ptr() + w_offset, dx.as_ptr() + 4 * x_offset
+    if by_name is not None:
+        kern.launch_by_name(stream, by_name, dy, wp, xp)
+    else:
+        kern.launch(stream, dy, wp, xp)
+    stream.synchronize()
+    return dy.copy_to_host()[:n]
+
+
+def gpu_gemm(gpu, fmt: str, buf: np.ndarray, a: np.ndarray, m: int, n: int, k: int, *, by_name=None) -> np.ndarray:
+    ctx, stream = gpu
+    dw = t.GpuBuffer.from_host(ctx, np.ascontiguousarray(buf, np.uint8).reshape(-1))
+    da = t.GpuBuffer.from_host(ctx, np.ascontiguousarray(a, np.float32).reshape(-1))
+    dc = t.GpuBuffer.from_host(ctx, np.full(max(m * n, 1), np.nan, np.float32))
+    kern = GEMM_KERNEL[fmt](m, n, k)
+    if by_name is not None:
+        kern.launch_by_name(stream, by_name, da, dw, dc)
+    else:
+        kern.launch(stream, da, dw, dc)
+    stream.synchronize()
+    return dc.copy_to_host()[: m * n].reshape(m, n)

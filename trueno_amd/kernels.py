@@ -1,0 +1,201 @@
+"""Host mirror of the k-quant kernel types of trueno-gpu/src/kernels/quantize.rs.
+
+Constructors, field names, `name()` strings and kernel parameter order are the reference's.
+`emit_ptx/build_ptx/as_module` (kernels/mod.rs:47-102) have no meaning without a PTX backend;
+their place is taken by `launch_config()` (the reference's documented geometry, kept for callers
+that build a LaunchConfig themselves - the library substitutes the kernel's real geometry) and
+`launch()` (the typed C-ABI launcher).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+
+from . import _ffi
+from .driver import CudaModule, CudaStream, GpuBuffer, GpuError, LaunchConfig, _check, _lib
+
+# quantize.rs:34-53
+Q4K_BLOCK_SIZE = 32
+Q4K_SUPER_BLOCK_SIZE = 256
+Q4K_SUPER_BLOCK_BYTES = 144
+Q4K_BLOCK_BYTES = 18
+Q5K_SUPER_BLOCK_SIZE = 256
+Q5K_SUPER_BLOCK_BYTES = 176
+Q6K_SUPER_BLOCK_SIZE = 256
+Q6K_SUPER_BLOCK_BYTES = 210
+
+
+class Q4KFormat(enum.Enum):
+    """quantize.rs:56-62."""
+    Simplified = 0
+    GgmlSuperBlock = 1
+
+
+class Kernel:
+    """kernels/mod.rs:47-102 (the part that survives without PTX)."""
+
+    def name(self) -> str:
+        raise NotImplementedError
+
+    def launch_config(self) -> LaunchConfig:
+        raise NotImplementedError
+
+
+def _ptr(b) -> int:
+    return b.as_ptr() if isinstance(b, GpuBuffer) else int(b)
+
+
+class _GemvKernel(Kernel):
+    _NAME = ""
+    _SB_BYTES = 0
+    _LAUNCHER = ""
+
+    def __init__(self, k: int, n: int):
+        """k first, then n (quantize.rs:1171-1173)."""
+        self.k = int(k)
+        self.n = int(n)
+
+    def name(self) -> str:
+        return self._NAME
+
+    def num_super_blocks_per_row(self) -> int:
+        return self.k // 256
+
+    def weight_bytes(self) -> int:
+        return self.n * self.num_super_blocks_per_row() * self._SB_BYTES
+
+    def launch_config(self) -> LaunchConfig:
+        """grid = N blocks, block = 32 threads, no shared memory (quantize.rs:1151-1155)."""
+        return LaunchConfig((self.n, 1, 1), (32, 1, 1), 0)
+
+    def kernel_args(self, y, w, x):
+        """(y_ptr, w_ptr, x_ptr, k_dim, n_dim) - quantize.rs:1190-1194."""
+        return [C.c_uint64(_ptr(y)), C.c_uint64(_ptr(w)), C.c_uint64(_ptr(x)), C.c_uint32(self.k), C.c_uint32(self.n)]
+
+    def launch(self, stream: CudaStream, y, w, x) -> None:
+        fn = getattr(_lib(), self._LAUNCHER)
+        _check(fn(stream.raw() if stream is not None else None, _ptr(y), _ptr(w), _ptr(x), self.k, self.n),
+               "KernelLaunch", self._NAME)
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, y, w, x) -> None:
+        """The reference's call shape: launch_kernel(module, name, LaunchConfig, args)."""
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(y, w, x))
+
+
+class Q4KGemvKernel(_GemvKernel):
+    """quantize.rs:1156-1523."""
+    _NAME = "q4k_gemv_warp_reduce"
+    _SB_BYTES = Q4K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q4k_gemv"
+
+
+class Q5KGemvKernel(_GemvKernel):
+    """quantize.rs:1532-1724."""
+    _NAME = "q5k_gemv_warp_reduce"
+    _SB_BYTES = Q5K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q5k_gemv"
+
+
+class Q6KGemvKernel(_GemvKernel):
+    """quantize.rs:1733-1965."""
+    _NAME = "q6k_gemv_warp_reduce"
+    _SB_BYTES = Q6K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q6k_gemv"
+
+
+class _GemmKernel(Kernel):
+    _NAME = ""
+    _SB_BYTES = 0
+    _LAUNCHER = ""
+
+    def __init__(self, m: int, n: int, k: int):
+        self.m, self.n, self.k = int(m), int(n), int(k)
+        self.tile_size = 32
+
+    def name(self) -> str:
+        return self._NAME
+
+    def with_tile_size(self, tile_size: int):
+        self.tile_size = int(tile_size)
+        return self
+
+    def num_super_blocks_per_row(self) -> int:
+        return self.k // 256
+
+    def weight_bytes(self) -> int:
+        return self.n * self.num_super_blocks_per_row() * self._SB_BYTES
+
+    def launch_config(self) -> LaunchConfig:
+        """tile_size^2 threads per block, one block per output tile (quantize.rs:376-386)."""
+        t = self.tile_size
+        return LaunchConfig(((self.n + t - 1) // t, (self.m + t - 1) // t, 1), (t * t, 1, 1), 0)
+
+    def kernel_args(self, a, b_quant, c):
+        """(a_ptr, b_quant_ptr, c_ptr, m, n, k) - quantize.rs:354-359."""
+        return [C.c_uint64(_ptr(a)), C.c_uint64(_ptr(b_quant)), C.c_uint64(_ptr(c)),
+                C.c_uint32(self.m), C.c_uint32(self.n), C.c_uint32(self.k)]
+
+    def launch(self, stream: CudaStream, a, b_quant, c) -> None:
+        fn = getattr(_lib(), self._LAUNCHER)
+        _check(fn(stream.raw() if stream is not None else None, _ptr(a), _ptr(b_quant), _ptr(c), self.m, self.n, self.k),
+               "KernelLaunch", self._NAME)
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, a, b_quant, c) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(a, b_quant, c))
+
+
+class QuantizeKernel(_GemmKernel):
+    """quantize.rs:66-147.  `QuantizeKernel.ggml(m, n, k)` is the 144-byte super-block format;
+    the plain constructor is the legacy 18-byte "simplified" format, which this backend does not
+    implement (launch raises)."""
+    _SB_BYTES = Q4K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q4k_gemm"
+
+    def __init__(self, m: int, n: int, k: int):
+        super().__init__(m, n, k)
+        self.block_size = Q4K_BLOCK_SIZE
+        self.format = Q4KFormat.Simplified
+
+    @staticmethod
+    def ggml(m: int, n: int, k: int) -> "QuantizeKernel":
+        kern = QuantizeKernel(m, n, k)
+        kern.block_size = Q4K_SUPER_BLOCK_SIZE
+        kern.format = Q4KFormat.GgmlSuperBlock
+        return kern
+
+    def name(self) -> str:
+        return "q4k_gemm_ggml" if self.format is Q4KFormat.GgmlSuperBlock else "q4k_gemm_fused"
+
+    def num_blocks_per_row(self) -> int:
+        return self.k // self.block_size
+
+    def launch(self, stream, a, b_quant, c) -> None:
+        if self.format is not Q4KFormat.GgmlSuperBlock:
+            raise GpuError("KernelLaunch", "q4k_gemm_fused (18-byte simplified blocks) is not provided by this backend")
+        super().launch(stream, a, b_quant, c)
+
+    def launch_by_name(self, stream, module, a, b_quant, c) -> None:
+        if self.format is not Q4KFormat.GgmlSuperBlock:
+            raise GpuError("FunctionNotFound", "CUDA function 'q4k_gemm_fused' not found in module")
+        super().launch_by_name(stream, module, a, b_quant, c)
+
+
+class Q5KKernel(_GemmKernel):
+    """quantize.rs:598-866."""
+    _NAME = "q5k_gemm_ggml"
+    _SB_BYTES = Q5K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q5k_gemm"
+
+
+class Q6KKernel(_GemmKernel):
+    """quantize.rs:884-1121."""
+    _NAME = "q6k_gemm_ggml"
+    _SB_BYTES = Q6K_SUPER_BLOCK_BYTES
+    _LAUNCHER = "trn_q6k_gemm"
+
+
+def dequant_f32(fmt: str, stream: CudaStream, out, w, n_sb: int, policy: int = 0) -> None:
+    """Test surface: out[sb*256+i] = weight i of super-block sb (policy 0 GEMV family, 1 GEMM family)."""
+    fn = getattr(_lib(), f"trn_{fmt}_dequant_f32")
+    _check(fn(stream.raw() if stream is not None else None, _ptr(out), _ptr(w), int(n_sb), int(policy)),
+           "KernelLaunch", f"{fmt}_dequant_f32")
