@@ -119,6 +119,21 @@ TRN_API trn_status trn_q4k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
 TRN_API trn_status trn_q5k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 
+/* A list of GEMVs issued with one call, in order, on one stream: the weight pass of a decode step
+ * (the caller in the reference issues one launch_kernel per matrix per token, docs/roadmaps/
+ * roadmap.yaml:359-368).  Entry i computes y = dequant(W) x exactly as the typed launcher of its
+ * format would; entry i+1 may read what entry i wrote.  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K. */
+typedef struct trn_gemv_desc {
+  uint32_t fmt;
+  uint32_t k;
+  uint32_t n;
+  uint32_t reserved;   /* must be 0 */
+  trn_dptr y;
+  trn_dptr w;
+  trn_dptr x;
+} trn_gemv_desc;
+TRN_API trn_status trn_kquant_gemv_batch(trn_stream stream, const trn_gemv_desc* descs, uint32_t count);
+
 /* ---- 9. test surface: dequantise to f32 (no counterpart in the reference) ------------------------
  * out[sb*256 + i] = weight i of super-block sb.  policy 0 = GEMV-family decode
  * (quantize.rs:1237-1483, :1589-1693, :1806-1934); policy 1 = GEMM-family decode as written

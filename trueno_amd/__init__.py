@@ -13,5 +13,5 @@ There is no CPU path: without libtrueno_hip.so or without a GPU every device cal
 from . import _ffi  # noqa: F401
 from .driver import (CudaContext, CudaModule, CudaStream, GpuBuffer, GpuError, LaunchConfig,  # noqa: F401
                      cuda_available, device_count)
-from .kernels import (Kernel, Q4KFormat, Q4KGemvKernel, Q5KGemvKernel, Q5KKernel, Q6KGemvKernel,  # noqa: F401
+from .kernels import (GemvBatch, Kernel, Q4KFormat, Q4KGemvKernel, Q5KGemvKernel, Q5KKernel, Q6KGemvKernel,  # noqa: F401
                       Q6KKernel, QuantizeKernel)

@@ -48,6 +48,7 @@ SIGNATURES = {
     "trn_q4k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q5k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q6k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
+    "trn_kquant_gemv_batch": [vp, vp, C.c_uint32],
     "trn_q4k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q5k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q6k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
@@ -63,6 +64,12 @@ SIGNATURES = {
     "trn_set_tuning": [C.c_char_p, C.c_int],
 }
 _RESTYPE = {"trn_error_name": C.c_char_p, "trn_error_string": C.c_char_p}
+
+
+class GemvDesc(C.Structure):
+    """trn_gemv_desc"""
+    _fields_ = [("fmt", C.c_uint32), ("k", C.c_uint32), ("n", C.c_uint32), ("reserved", C.c_uint32),
+                ("y", C.c_uint64), ("w", C.c_uint64), ("x", C.c_uint64)]
 
 
 class LibraryMissing(OSError):

@@ -126,7 +126,7 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
 #define KQ_GEMV_KERNELS(fmtname, FMT)                                                                    \
   extern "C" __global__ void __launch_bounds__(512)                                                      \
       fmtname##_gemv_warp_reduce(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim) {     \
-    gemv_fast_body<FMT, 4>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x);                                \
+    gemv_fast_body<FMT, 2>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x);                                \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim) {         \
@@ -146,7 +146,7 @@ KQ_GEMV_KERNELS(q6k, FMT_Q6K)
   extern "C" __global__ void __launch_bounds__(512)                                                      \
       fmtname##_gemm_ggml(const float* a, const uint8_t* b_quant, float* c, u32 m, u32 n, u32 k) {       \
     for (u32 r = blockIdx.y; r < m; r += gridDim.y) {                                                    \
-      gemv_fast_body<FMT, 4>(c + static_cast<size_t>(r) * n, b_quant, a + static_cast<size_t>(r) * k,    \
+      gemv_fast_body<FMT, 2>(c + static_cast<size_t>(r) * n, b_quant, a + static_cast<size_t>(r) * k,    \
                              k, n, blockIdx.x, gridDim.x);                                               \
       __syncthreads();                                                                                   \
     }                                                                                                    \

@@ -43,7 +43,7 @@ const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2 };
 
 constexpr int kMaxDevices = 64;
-constexpr uint32_t kGemvRowsPerBatch = 4;     // U of the fast GEMV kernel
+constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 
 struct DeviceKernels {
@@ -129,7 +129,7 @@ GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n) {
   uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : std::max<uint32_t>(1u, 4u / sw);
   groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
   const uint32_t ug = kGemvRowsPerBatch * groups;
-  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : 3u;
+  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : 4u;
   const uint64_t target_blocks = uint64_t(d.cu_count) * per_cu;
   uint64_t rows = (uint64_t(n) + target_blocks - 1) / target_blocks;
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
@@ -460,6 +460,19 @@ trn_status trn_q5k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
 }
 trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
   return st(launch_gemm_like(Q6K, static_cast<hipStream_t>(s), a, b, c, m, n, k, false));
+}
+
+trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {
+  if (count == 0) return TRN_SUCCESS;
+  if (!descs) return TRN_ERROR_INVALID_VALUE;
+  for (uint32_t i = 0; i < count; ++i)  // validate the whole list before anything is launched
+    if (descs[i].fmt < 4 || descs[i].fmt > 6 || descs[i].reserved != 0 || descs[i].k % 256u != 0) return TRN_ERROR_INVALID_VALUE;
+  for (uint32_t i = 0; i < count; ++i) {
+    const trn_gemv_desc& d = descs[i];
+    hipError_t e = launch_gemm_like(Fmt(d.fmt - 4), static_cast<hipStream_t>(s), d.x, d.w, d.y, 1, d.n, d.k, true);
+    if (e != hipSuccess) return st(e);
+  }
+  return TRN_SUCCESS;
 }
 
 // ---- 9. dequantise test surface ----------------------------------------------------------

@@ -199,3 +199,29 @@ def dequant_f32(fmt: str, stream: CudaStream, out, w, n_sb: int, policy: int = 0
     fn = getattr(_lib(), f"trn_{fmt}_dequant_f32")
     _check(fn(stream.raw() if stream is not None else None, _ptr(out), _ptr(w), int(n_sb), int(policy)),
            "KernelLaunch", f"{fmt}_dequant_f32")
+
+
+class GemvBatch:
+    """An ordered list of k-quant GEMVs issued with one library call (trn_kquant_gemv_batch): the
+    weight pass of one decode step.  Entries run in order on the stream; a later entry may read an
+    earlier entry's output."""
+
+    _FMT = {"q4k": 4, "q5k": 5, "q6k": 6}
+
+    def __init__(self):
+        self._entries = []
+        self._array = None
+
+    def add(self, fmt: str, k: int, n: int, y, w, x) -> "GemvBatch":
+        self._entries.append(_ffi.GemvDesc(self._FMT[fmt], int(k), int(n), 0, _ptr(y), _ptr(w), _ptr(x)))
+        self._array = None
+        return self
+
+    def __len__(self) -> int:
+        return len(self._entries)
+
+    def launch(self, stream: CudaStream) -> None:
+        if self._array is None:
+            self._array = (_ffi.GemvDesc * len(self._entries))(*self._entries)
+        _check(_lib().trn_kquant_gemv_batch(stream.raw() if stream is not None else None, self._array, len(self._entries)),
+               "KernelLaunch", "kquant_gemv_batch")
