@@ -4,12 +4,12 @@
 A step is one 7B-style decode weight pass: 32 layers x {Q,K,V,O: Q4_K 4096x4096; gate, up: Q4_K
 11008x4096; down: Q6_K 4096x11008} plus the Q6_K 32000x4096 head - 225 GEMVs over 4.12 GB of
 distinct, seeded synthetic weights resident in HBM (far beyond the 256 MB Infinity Cache, so every
-pass streams from HBM).  The GEMVs of a pass are issued in order on one stream; within a layer
-Q, K, V, O, gate, up read the layer's activation vector x_l ~ N(0,1) (4096) and down reads a second
-N(0,1) vector (11008).  `value` is algorithmic bytes (weights + x + y, each once) over wall time.
+pass streams from HBM).  The GEMVs form a dependent chain as in a decoder: q,k,v <- h; o <- q;
+gate,up <- o; down <- gate; next h <- down; head <- h, with h0 ~ N(0,1) and every input
+RMS-normalised.  The list goes to the library in one call (trn_kquant_gemv_batch).  `value` is algorithmic bytes (weights + x + y, each once) over wall time.
 
-Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (Q4_K GEMV: 2.83 of the
-4.12 GB), timed per launch with HIP events on the launch stream; `cpu_baseline`: the CPU port
+Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (the Q4_K GEMV: 192 of the
+225 launches, 2.84 of the 4.13 GB), its launches of one pass timed with HIP events on their stream; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.
 """
 import argparse
@@ -25,6 +25,11 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per q4k_gemv_flags launch, averaged over the 192 Q4_K launches of the full pass: rocprofv3
+# FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the counter reads for kq_copy_u128 on
+# 256 MiB (profiles/kquant_gemv_hbm_traffic_pmc.md).  Counters cannot be read from inside this
+# process, so the figure is carried here and re-measured whenever the kernel changes.
+Q4K_GEMV_TRAFFIC_BYTES_PER_LAUNCH = 14_995_230
 LAYERS = 32
 SB = {"q4k": 144, "q5k": 176, "q6k": 210}
 LAYER_MATS = [("q", "q4k", 4096, 4096), ("k", "q4k", 4096, 4096), ("v", "q4k", 4096, 4096), ("o", "q4k", 4096, 4096),
@@ -42,6 +47,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-executors", action="store_true", help="skip the comparison runs of the opt-in one-launch executors")
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -77,69 +83,104 @@ def main() -> int:
     ys = {name: t.GpuBuffer(ctx, n, np.float32) for name, _, n, _ in LAYER_MATS}
     print(f"[bench] generated and uploaded {layers} layers in {time.time() - t_gen:.1f} s", file=sys.stderr, flush=True)
 
+    # ---- the pass as one dependent list: per layer  q,k,v <- h ; o <- q ; gate,up <- o ; down <- gate ;
+    #      next h = down ; head <- h.  Every entry normalises its input (RMS, no gain), which keeps the
+    #      chain of random matrices in range.
+    NORM = t.GemvBatch.NORM_INPUT
+    act = {nm: t.GpuBuffer(ctx, n, np.float32) for nm, n in (("q", 4096), ("k", 4096), ("v", 4096), ("o", 4096),
+                                                             ("gate", 11008), ("up", 11008), ("down", 4096))}
+    h0 = xs[0][0]
+    logits = y[32000]
+    src_of = {"q": None, "k": None, "v": None, "o": "q", "gate": "o", "up": "o", "down": "gate"}
     batch = t.GemvBatch()
-    q4_batch = t.GemvBatch()
-    total_bytes = q4_bytes = 0
+    total_bytes = 0
+    weight_bytes = 0
+    h = h0
     for layer in range(layers):
-        x4096, x11008 = xs[layer]
         for name, fmt, n, k in LAYER_MATS:
-            x = x11008 if k == 11008 else x4096
-            batch.add(fmt, k, n, ys[name], weights[layer][name], x)
+            x = h if src_of[name] is None else act[src_of[name]]
+            batch.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
             total_bytes += alg_bytes(fmt, n, k)
-            if fmt == "q4k":
-                q4_batch.add(fmt, k, n, ys[name], weights[layer][name], x)
-                q4_bytes += alg_bytes(fmt, n, k)
-    batch.add(HEAD[1], HEAD[3], HEAD[2], y[32000], head_w, xs[-1][0])
+            weight_bytes += n * (k // 256) * SB[fmt]
+        h = act["down"]
+    batch.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, h, NORM)
     total_bytes += alg_bytes(HEAD[1], HEAD[2], HEAD[3])
+    weight_bytes += HEAD[2] * (HEAD[3] // 256) * SB[HEAD[1]]
 
     def ev():
         e = C.c_void_p()
         assert L.trn_event_create(C.byref(e)) == 0
         return e
 
+    # one plain copy of known size (256 MiB read + 256 MiB written): the yardstick that profiler byte
+    # counters of the same run are scaled by
+    cal_src = t.GpuBuffer(ctx, 64 << 20, np.float32)
+    cal_dst = t.GpuBuffer(ctx, 64 << 20, np.float32)
+    assert L.trn_copy_u128(stream.raw(), cal_dst.as_ptr(), cal_src.as_ptr(), 256 << 20) == 0
+    stream.synchronize()
+    cal_src.free()
+    cal_dst.free()
+
     def elapsed_ms(a, b):
         ms = C.c_float()
         assert L.trn_event_elapsed_ms(C.byref(ms), a, b) == 0
         return float(ms.value)
 
-    # ---- timed region: W warm-up passes, then exactly K passes ------------------------------------
-    for _ in range(args.warmup):
-        batch.launch(stream)
-    stream.synchronize()
-    e0, e1 = ev(), ev()
-    t0 = time.perf_counter()
-    L.trn_event_record(e0, stream.raw())
-    for _ in range(args.steps):
-        batch.launch(stream)
-    L.trn_event_record(e1, stream.raw())
-    stream.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = elapsed_ms(e0, e1)
-    ms_per_step = wall_ms / args.steps
-    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+    def run_passes(steps, warmup):
+        for _ in range(warmup):
+            batch.launch(stream)
+        stream.synchronize()
+        e0, e1 = ev(), ev()
+        t0 = time.perf_counter()
+        L.trn_event_record(e0, stream.raw())
+        for _ in range(steps):
+            batch.launch(stream)
+        L.trn_event_record(e1, stream.raw())
+        stream.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        return wall / steps, elapsed_ms(e0, e1) / steps
 
-    # ---- dominant kernel (Q4_K GEMV), per launch, HIP events on the launch stream ------------------
-    n_q4 = len(q4_batch)
-    evs = [ev() for _ in range(n_q4 + 1)]
-    one = []
+    # ---- timed region: W warm-up passes, then exactly K passes (one cooperative launch per pass) ----
+    ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup)
+    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+    assert np.all(np.isfinite(logits.copy_to_host())), "the pass produced non-finite logits"
+
+    # ---- dominant kernel: the Q4_K GEMV (192 of the 225 launches, 2.84 of the 4.13 GB).  Its launches of one
+    #      pass, in pass order, back to back on the stream, bracketed by HIP events on that stream.
+    q4 = t.GemvBatch()
+    q4_bytes = 0
+    h = h0
     for layer in range(layers):
         for name, fmt, n, k in LAYER_MATS:
             if fmt == "q4k":
-                one.append(t.GemvBatch().add(fmt, k, n, ys[name], weights[layer][name], xs[layer][0]))
-    durations = []
-    for rep in range(3):
+                x = h if src_of[name] is None else act[src_of[name]]
+                q4.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
+                q4_bytes += alg_bytes(fmt, n, k)
+        h = act["down"]
+    n_q4 = len(q4)
+    e0, e1 = ev(), ev()
+    q4_ms = []
+    for _ in range(5):
+        q4.launch(stream)
         stream.synchronize()
-        L.trn_event_record(evs[0], stream.raw())
-        for i, b in enumerate(one):
-            b.launch(stream)
-            L.trn_event_record(evs[i + 1], stream.raw())
+        L.trn_event_record(e0, stream.raw())
+        q4.launch(stream)
+        L.trn_event_record(e1, stream.raw())
         stream.synchronize()
-        durations.append(sum(elapsed_ms(evs[i], evs[i + 1]) for i in range(n_q4)) / n_q4)
-    q4_ms = min(durations)
+        q4_ms.append(elapsed_ms(e0, e1) / n_q4)
+    q4_ms = sorted(q4_ms)[len(q4_ms) // 2]
     q4_bytes_per_launch = q4_bytes / n_q4
     achieved = q4_bytes_per_launch / (q4_ms * 1e-3) / 1e9
 
-    # ---- per-shape steady-state table (cold: rotates through the 32 layers' copies) ----------------
+    # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
+    other_modes = {}
+    for mode, label in (() if args.no_executors else ((1, "resident_workgroups"), (2, "streaming_producer"))):
+        L.trn_set_tuning(b"batch_mode", mode)
+        ms, _ = run_passes(max(3, args.steps // 2), 1)
+        other_modes[label] = round(ms * 1e3, 1)
+    L.trn_set_tuning(b"batch_mode", 0)
+
+    # ---- per-shape single-launch table (cold: rotates through the layers' copies) -----------------------
     shapes = {}
     for name, fmt, n, k in LAYER_MATS[3:] + [HEAD]:
         b = t.GemvBatch()
@@ -181,20 +222,24 @@ def main() -> int:
                          f"dequantise-row + AVX2 dot, {'AVX2+FMA' if cb.has_avx2() else 'scalar'}"}
 
     out = {
-        "metric": "k-quant GEMV achieved HBM GB/s over a 7B decode weight pass",
+        "metric": "k-quant GEMV achieved HBM GB/s (% of peak) + \u00b5s per 7B decode weight pass",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"7B-style decode weight pass: {layers} layers x (4x Q4_K 4096x4096 + 2x Q4_K 11008x4096 + "
-                               f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} GEMVs, {total_bytes / 1e9:.3f} GB, "
-                               "batch 1, f32 x and y", "gemvs": len(batch), "bytes_per_step": total_bytes},
+                               f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} dependent GEMVs "
+                               f"(q,k,v<-h; o<-q; gate,up<-o; down<-gate; h<-down), {total_bytes / 1e9:.3f} GB, batch 1, "
+                               "f32 x and y, RMS-normalised inputs", "gemvs": len(batch), "bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "q4k_gemv_warp_reduce", "launches": n_q4,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": Q4K_GEMV_TRAFFIC_BYTES_PER_LAUNCH if layers == LAYERS else None,
+                     "kernel": "q4k_gemv_flags", "launches_per_pass": n_q4,
                      "bytes_per_launch": round(q4_bytes_per_launch), "us_per_launch": round(q4_ms * 1e3, 3)},
         "cpu_baseline": cpu,
         "extra": {"us_per_pass": round(ms_per_step * 1e3, 1), "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-                  "gpu_event_ms_per_step": round(gpu_ms / args.steps, 4), "per_shape_cold": shapes,
+                  "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
+                  "us_per_pass_one_launch_executors": other_modes,
+                  "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }
     print(json.dumps(out), flush=True)

@@ -122,12 +122,22 @@ TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
 /* A list of GEMVs issued with one call, in order, on one stream: the weight pass of a decode step
  * (the caller in the reference issues one launch_kernel per matrix per token, docs/roadmaps/
  * roadmap.yaml:359-368).  Entry i computes y = dequant(W) x exactly as the typed launcher of its
- * format would; entry i+1 may read what entry i wrote.  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K. */
+ * format would; a later entry may read what an earlier one wrote (the library finds those
+ * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
+ * By default the list is issued as one launch per entry.  With trn_set_tuning("batch_mode", 1 or 2),
+ * and when every entry meets the fast kernels' alignment (x 16 B, W 16 B / 2 B for Q6_K), the list
+ * runs as ONE cooperative launch of resident workgroups with device-side barriers at the
+ * dependencies.  That form keeps, per (device, stream), a small device buffer with the list and its
+ * barrier counters (allocated on first use, kept until the process ends); a list identical to the
+ * previous one on that stream is not uploaded again.  If a device-side wait ever runs out of its
+ * (seconds-long) spin budget the kernel exits and the next call on that stream returns
+ * hipErrorLaunchFailure (719).  All three forms give bit-identical results. */
+#define TRN_GEMV_NORM_INPUT 1u /* the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x */
 typedef struct trn_gemv_desc {
   uint32_t fmt;
   uint32_t k;
   uint32_t n;
-  uint32_t reserved;   /* must be 0 */
+  uint32_t flags;      /* 0 or TRN_GEMV_NORM_INPUT */
   trn_dptr y;
   trn_dptr w;
   trn_dptr x;
@@ -155,7 +165,12 @@ TRN_API const char* trn_error_name(trn_status status);
 TRN_API const char* trn_error_string(trn_status status);
 /* Number of compute units of the current device (sizes the launches). */
 TRN_API trn_status trn_device_cu_count(int* count);
-/* Launch tuning knobs, process-wide: "gemv_blocks_per_cu", "gemv_row_groups".  0 restores the default. */
+/* Launch tuning knobs, process-wide; 0 restores the default.  "gemv_blocks_per_cu", "gemv_row_groups":
+ * geometry of the single-GEMV kernels.  "batch_mode": how trn_kquant_gemv_batch runs a list - 0 one
+ * launch per entry (default), 1 one cooperative launch of resident workgroups with device-side
+ * barriers, 2 as 1 with a producer wave per CU streaming the weights through an LDS ring.
+ * "chain_blocks_per_cu", "chain_waves", "chain_prefetch_off", "stream_consumers": geometry of modes 1/2.
+ * "chain_spin_limit": polls a device-side barrier wait may take before it gives up. */
 TRN_API trn_status trn_set_tuning(const char* key, int value);
 
 #ifdef __cplusplus

@@ -1,0 +1,263 @@
+// Persistent executor for an ordered list of k-quant GEMVs (the weight pass of one decode step).
+//
+// Issued one kernel per matrix, a pass is bound by per-launch latency, not by HBM: each launch pays
+// a dispatch gap, an activation-staging phase and a first-load latency during which HBM idles, and a
+// 4096x4096 Q4_K matrix is only ~1.5 us of streaming.  Here the whole list runs in ONE cooperative
+// launch whose workgroups all stay resident:
+//   * every workgroup owns a fixed share of the rows of every entry;
+//   * where an entry reads what an earlier entry wrote, the host marks a device-wide barrier in front
+//     of it; entries between two barriers are independent and stream back to back;
+//   * weights do not depend on activations, so before a workgroup waits at a barrier it has already
+//     requested the first rows of the next entry - HBM keeps streaming across the dependency;
+//   * the barrier is a (two-level) counter in device memory: atomic add to arrive, bounded spin to
+//     leave.  A spin that runs out sets a status word and every workgroup exits; nothing can hang.
+//   * the only data that crosses workgroups are the activation vectors and the counters.  The L2s of
+//     the eight XCDs are not coherent with each other for ordinary accesses, and the release/acquire
+//     fences that would make them so write back / invalidate whole caches (tens of microseconds per
+//     barrier, measured).  Instead exactly those accesses are made coherent: y is stored and x is
+//     loaded with agent-scope atomic (relaxed) accesses, which go to the memory side; weights are
+//     read-only and keep the fast path.
+// The per-row arithmetic is the quarter-block engine of kquant_quarter.hip.h, unchanged.
+//
+// CHAIN_NORM_INPUT: the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x (an RMS normalisation
+// without gain, applied as one factor on y; every workgroup stages all of x anyway).  It keeps a
+// chain of random matrices in range; the reference has it as a separate kernel
+// (trueno-gpu/src/kernels/layernorm.rs:388-470).
+#pragma once
+#include "kquant_quarter.hip.h"
+
+#ifdef CHAIN_TS
+extern __device__ unsigned long long* g_chain_ts;   // [entry][4] for workgroup CHAIN_TS_WG: start, after wait, after x, end
+#define CHAIN_STAMP(slot) do { if (g_chain_ts && blockIdx.x == g_chain_ts_wg && threadIdx.x == 0) g_chain_ts[4 * g_chain_ts_entry + (slot)] = wall_clock64(); } while (0)
+extern __device__ unsigned g_chain_ts_wg;
+static __device__ unsigned g_chain_ts_entry;
+#else
+#define CHAIN_STAMP(slot) do { } while (0)
+#endif
+
+struct ChainEntry {
+  u32 fmt, k, n, flags;
+  const uint8_t* w;
+  const float* x;
+  float* y;
+};
+enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u };
+constexpr float kChainNormEps = 1e-6f;
+
+// Sum of squares of the activation vector in ONE fixed order, whatever the launch shape: lane l adds
+// the 16-byte units l, l+64, l+128, ... (x, y, z, w in turn), then the fixed wave butterfly.  Every
+// wave computes it for itself from the staged copy, so no kernel's result depends on its geometry.
+template <class Q>
+__device__ __forceinline__ float canonical_sumsq_lds(const f32x4* lds4, u32 units, u32 lane) {
+  float ss = 0.0f;
+  for (u32 u = lane; u < units; u += 64u) {
+    const f32x4 v = lds4[Q::swz(u)];
+    ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+  }
+  return wave_sum(ss);
+}
+
+// Barrier counters.  Every workgroup adding to one address costs ~15 ns per add at the memory side
+// (8 us for 512 workgroups, measured); arrival is therefore two-level: workgroups arrive at the
+// counter of their group of 32, the last one of a group arrives at the top counter, everybody polls
+// the top counter (~1.5 us per barrier at 256 workgroups).  One barrier owns kChainBarrierStride
+// words: word 0 is the top counter, word 64*(1+g) the counter of group g (each on its own 256 bytes).
+constexpr u32 kChainGroup = 32u;
+__host__ __device__ constexpr u32 chain_barrier_stride(u32 num_workgroups) {
+  return 64u * (1u + (num_workgroups + kChainGroup - 1u) / kChainGroup);
+}
+
+__device__ __forceinline__ void chain_arrive(u32* barrier) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this thread's coherent y stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const u32 grp = blockIdx.x / kChainGroup;
+    const u32 gsize = min(kChainGroup, gridDim.x - grp * kChainGroup);
+    const u32 old = __hip_atomic_fetch_add(barrier + 64u * (1u + grp), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == gsize - 1u) __hip_atomic_fetch_add(barrier, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// true when every group has arrived; false when the spin budget ran out
+__device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* status, u32* s_flag) {
+  if (threadIdx.x == 0) {
+    const u32 target = (gridDim.x + kChainGroup - 1u) / kChainGroup;
+    u32 spins = 0, ok = 1u;
+    while (__hip_atomic_load(barrier, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      __builtin_amdgcn_s_sleep(4);
+      if (++spins > spin_limit) {
+        ok = 0u;
+        __hip_atomic_fetch_or(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        break;
+      }
+    }
+    *s_flag = ok;
+  }
+  __syncthreads();
+  return *s_flag != 0u;
+}
+
+// Touches one dword in every 128-byte line of this workgroup's share of rows of entry `e` (capped),
+// so the lines are on their way into this XCD's L2 while the workgroup waits at a barrier or works
+// on the current entry.  The loaded words are returned so the loads stay live; the caller folds
+// them into a value it never stores.
+constexpr u32 kChainPrefetchLoads = 3u;         // per thread
+constexpr u32 kChainPrefetchLine = 128u;
+template <int U>
+__device__ __forceinline__ u32 chain_prefetch(const ChainEntry& e) {
+  const u32 nsb = e.k >> 8;
+  const u32 sbb = e.fmt == FMT_Q4K ? 144u : e.fmt == FMT_Q5K ? 176u : 210u;
+  u32 rows_per_block = (e.n + gridDim.x - 1) / gridDim.x;
+  rows_per_block = ((rows_per_block + U - 1) / U) * U;
+  const u32 row0 = blockIdx.x * rows_per_block;
+  if (row0 >= e.n || nsb == 0) return 0u;
+  const u32 rows = min(rows_per_block, e.n - row0);
+  const size_t row_bytes = static_cast<size_t>(nsb) * sbb;
+  const size_t bytes = static_cast<size_t>(rows) * row_bytes;
+  const uint8_t* base = e.w + static_cast<size_t>(row0) * row_bytes;
+  u32 acc = 0u;
+#pragma unroll
+  for (u32 i = 0; i < kChainPrefetchLoads; ++i) {
+    const size_t off = (static_cast<size_t>(i) * blockDim.x + threadIdx.x) * kChainPrefetchLine;
+    if (off + 4 <= bytes) acc ^= *reinterpret_cast<const u32*>(base + (off & ~static_cast<size_t>(3)));
+  }
+  return acc;
+}
+
+// One entry on this workgroup's share of rows.  Returns false if the barrier wait gave up.
+//   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][16 floats reduction scratch]
+// COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
+template <int FMT, int U, bool COHERENT = false>
+__device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
+                                           f32x4* lds4, u32* s_flag, const ChainEntry* next = nullptr, u32* sink = nullptr) {
+  using Q = Quarter<FMT>;
+  const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
+  const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
+  const u32 slabs = (nsb + 15u) >> 4;
+  const u32 sw_count = slabs < waves ? slabs : waves;
+  const u32 groups = waves / sw_count;
+  u32 rows_per_block = (n_dim + gridDim.x - 1) / gridDim.x;
+  rows_per_block = ((rows_per_block + U - 1) / U) * U;
+  const u32 row0 = blockIdx.x * rows_per_block;
+  const bool has_rows = row0 < n_dim && nsb != 0;
+  const u32 batches = has_rows ? rows_per_block / U : 0u;
+  const u32 sw = wave % sw_count, grp = wave / sw_count;
+  const bool wave_active = grp < groups && grp < batches;
+  const u32 sbl = lane >> 2, c = lane & 3u;
+  const size_t row_bytes = static_cast<size_t>(nsb) * Q::SB;
+
+  CHAIN_STAMP(0);
+  typename Q::Regs regs[U];
+  auto issue = [&](u32 slab, u32 b) {
+    const u32 sb = slab * 16u + sbl;
+    const u32 sbc = sb < nsb ? sb : nsb - 1;
+    const uint8_t* col = e.w + static_cast<size_t>(sbc) * Q::SB;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      u32 row = row0 + b * U + u;
+      row = row < n_dim ? row : n_dim - 1;
+      Q::load(regs[u], col + row * row_bytes, c);
+    }
+  };
+  if (wave_active) issue(sw, grp);          // in flight across the barrier and the activation staging
+  u32 touched = 0u;
+  if (next) touched = chain_prefetch<U>(*next);
+
+  if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
+  CHAIN_STAMP(1);
+  if (!has_rows) return true;
+
+  const u32 units = k_dim >> 2;
+  const f32x4* x4 = reinterpret_cast<const f32x4*>(e.x);
+  for (u32 u = tid; u < units; u += blockDim.x) {
+    f32x4 v;
+    if constexpr (COHERENT) {
+      const u32* xw = reinterpret_cast<const u32*>(e.x) + 4u * u;
+      v.x = __uint_as_float(__hip_atomic_load(xw + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      v.y = __uint_as_float(__hip_atomic_load(xw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      v.z = __uint_as_float(__hip_atomic_load(xw + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      v.w = __uint_as_float(__hip_atomic_load(xw + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    } else {
+      v = x4[u];
+    }
+    lds4[Q::swz(u)] = v;
+  }
+  float* part = reinterpret_cast<float*>(lds4 + units);
+  __syncthreads();
+  CHAIN_STAMP(2);
+  float scale = 1.0f;
+  if ((e.flags & CHAIN_NORM_INPUT) != 0u)
+    scale = 1.0f / sqrtf(canonical_sumsq_lds<Q>(lds4, units, lane) / static_cast<float>(k_dim) + kChainNormEps);
+
+  if (wave_active) {
+    for (u32 slab = sw; slab < slabs; slab += sw_count) {
+      const u32 sb = slab * 16u + sbl;
+      const bool valid = sb < nsb;
+      const u32 sbc = valid ? sb : nsb - 1;
+      float xr[64];
+      float sx[Q::NSUM];
+#pragma unroll
+      for (int s = 0; s < Q::NSUM; ++s) sx[s] = 0.0f;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const u32 unit = (256u * sbc + Q::value_index(c, 4 * q)) >> 2;
+        f32x4 v = lds4[Q::swz(unit)];
+        if (!valid) v = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+        sx[Q::sum_index(4 * q)] += (v.x + v.y) + (v.z + v.w);
+      }
+      for (u32 b = grp; b < batches; b += groups) {
+        if (slab != sw || b != grp) issue(slab, b);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
+          if (lane == 0) {
+            const u32 idx = sw * rows_per_block + b * U + u;
+            part[idx] = (slab == sw) ? p : part[idx] + p;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (u32 t = tid; t < rows_per_block; t += blockDim.x) {
+    const u32 row = row0 + t;
+    if (row < n_dim) {
+      float s = part[t];
+      for (u32 i = 1; i < sw_count; ++i) s += part[i * rows_per_block + t];
+      if constexpr (COHERENT)
+        __hip_atomic_store(reinterpret_cast<u32*>(e.y) + row, __float_as_uint(s * scale), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      else
+        e.y[row] = s * scale;
+    }
+  }
+  if (sink && touched == 0x9E3779B9u) *sink = touched;   // keeps the prefetch loads; practically never taken
+  CHAIN_STAMP(3);
+  return true;
+}
+
+template <int U>
+__device__ __forceinline__ void chain_body(const ChainEntry* __restrict__ entries, u32 count, u32* counters,
+                                           u32* status, u32 spin_limit, u32 prefetch) {
+  extern __shared__ f32x4 lds4[];
+  __shared__ u32 s_flag;
+  u32 bar = 0;
+  for (u32 i = 0; i < count; ++i) {
+#ifdef CHAIN_TS
+    if (threadIdx.x == 0 && blockIdx.x == g_chain_ts_wg) g_chain_ts_entry = i;
+#endif
+    const ChainEntry e = entries[i];
+    u32* wait_counter = (e.flags & CHAIN_BARRIER_BEFORE) ? counters + bar * chain_barrier_stride(gridDim.x) : nullptr;
+    bool ok = true;
+    const ChainEntry* next = (prefetch && i + 1 < count) ? entries + i + 1 : nullptr;
+    if (e.fmt == FMT_Q4K) ok = chain_step<FMT_Q4K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
+    else if (e.fmt == FMT_Q5K) ok = chain_step<FMT_Q5K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
+    else if (e.fmt == FMT_Q6K) ok = chain_step<FMT_Q6K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
+    if (!ok) return;
+    if (wait_counter) ++bar;
+    const bool arrive = i + 1 < count && (entries[i + 1].flags & CHAIN_BARRIER_BEFORE) != 0u;
+    if (arrive) chain_arrive(counters + bar * chain_barrier_stride(gridDim.x));
+    else __syncthreads();                  // LDS is reused by the next entry
+  }
+}

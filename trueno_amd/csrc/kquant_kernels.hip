@@ -8,92 +8,16 @@
 // 32-thread warp, :1151-1155): here it is a property of the kernel, chosen by the host library,
 // and every kernel gives the same result for any grid size and any block size that is a
 // multiple of 64.
-#include "kquant_quarter.hip.h"
+#include "kquant_chain.hip.h"
+#include "kquant_stream.hip.h"
 
-// ------------------------------------------------------------------------------------------
-// Fast GEMV body.  One workgroup owns R consecutive rows; the activation vector is staged once
-// into LDS (swizzled), then each wave keeps its 64-activations-per-lane slice in registers and
-// streams rows: U rows of loads in flight per wave, unpack in registers, factorised dot, wave
-// reduction.  K is cut in slabs of 16 super-blocks (one wave-width); with S slabs, min(S, waves)
-// waves share a row and their partial sums meet in LDS.
-//   dynamic LDS = K*4 bytes (activations) + Sw*R*4 bytes (partial sums)
-// ------------------------------------------------------------------------------------------
-template <int FMT, int U>
-__device__ __forceinline__ void gemv_fast_body(float* __restrict__ y, const uint8_t* __restrict__ w,
-                                               const float* __restrict__ x, u32 k_dim, u32 n_dim,
-                                               u32 block_id, u32 num_blocks) {
-  using Q = Quarter<FMT>;
-  extern __shared__ f32x4 lds4[];
-  const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
-  const u32 nsb = k_dim >> 8;
-  if (waves == 0 || nsb == 0 || n_dim == 0) return;
-  const u32 slabs = (nsb + 15u) >> 4;
-  const u32 sw_count = slabs < waves ? slabs : waves;  // waves sharing one row
-  const u32 groups = waves / sw_count;                 // row groups per workgroup
-  const u32 ug = U * groups;
-  u32 rows_per_block = (n_dim + num_blocks - 1) / num_blocks;
-  rows_per_block = ((rows_per_block + ug - 1) / ug) * ug;
-  const u32 row0 = block_id * rows_per_block;
-  if (row0 >= n_dim) return;
-
-  const u32 units = k_dim >> 2;
-  const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
-  for (u32 u = tid; u < units; u += blockDim.x) lds4[Q::swz(u)] = x4[u];
-  float* part = reinterpret_cast<float*>(lds4 + units);
-  __syncthreads();
-
-  const u32 sw = wave % sw_count, grp = wave / sw_count;
-  if (grp < groups) {
-    const u32 sbl = lane >> 2, c = lane & 3u;
-    const size_t row_bytes = static_cast<size_t>(nsb) * Q::SB;
-    const u32 batches = rows_per_block / ug;
-    for (u32 slab = sw; slab < slabs; slab += sw_count) {
-      const u32 sb = slab * 16u + sbl;
-      const bool valid = sb < nsb;
-      const u32 sbc = valid ? sb : nsb - 1;
-      float xr[64];
-      float sx[Q::NSUM];
-#pragma unroll
-      for (int s = 0; s < Q::NSUM; ++s) sx[s] = 0.0f;
-#pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const u32 unit = (256u * sbc + Q::value_index(c, 4 * q)) >> 2;
-        f32x4 v = lds4[Q::swz(unit)];
-        if (!valid) v = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
-        sx[Q::sum_index(4 * q)] += (v.x + v.y) + (v.z + v.w);
-      }
-      const uint8_t* col = w + static_cast<size_t>(sbc) * Q::SB;
-      for (u32 b = 0; b < batches; ++b) {
-        const u32 rl = (b * groups + grp) * U;
-        typename Q::Regs regs[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          u32 row = row0 + rl + u;
-          row = row < n_dim ? row : n_dim - 1;
-          Q::load(regs[u], col + row * row_bytes, c);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
-          if (lane == 0) {
-            const u32 idx = sw * rows_per_block + rl + u;
-            part[idx] = (slab == sw) ? p : part[idx] + p;
-          }
-        }
-      }
-    }
-  }
-  __syncthreads();
-  for (u32 t = tid; t < rows_per_block; t += blockDim.x) {
-    const u32 row = row0 + t;
-    if (row < n_dim) {
-      float s = part[t];
-      for (u32 i = 1; i < sw_count; ++i) s += part[i * rows_per_block + t];
-      y[row] = s;
-    }
-  }
-}
+// The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
+// activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
+// slice in registers and streams rows (U rows of 128-bit loads in flight per wave), unpacks in
+// registers, forms the factorised dot product and reduces across the wave with DPP.  K is cut in
+// slabs of 16 super-blocks (one wave-width); with S slabs, min(S, waves) waves share a row and
+// their partial sums meet in LDS.
+//   dynamic LDS = K*4 (activations) + Sw*R*4 (partial sums) + 64 bytes
 
 // ------------------------------------------------------------------------------------------
 // Generic GEMV body: one wave per row, byte loads only.  Any pointer alignment, any K that is
@@ -102,11 +26,20 @@ __device__ __forceinline__ void gemv_fast_body(float* __restrict__ y, const uint
 template <int FMT, int POLICY>
 __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const uint8_t* __restrict__ w,
                                                   const float* __restrict__ x, u32 k_dim, u32 n_dim,
-                                                  u32 block_id, u32 num_blocks) {
+                                                  u32 block_id, u32 num_blocks, u32 flags) {
   constexpr u32 SB = sb_bytes<FMT>::value;
   const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
   if (waves == 0) return;
   const u32 nsb = k_dim >> 8;
+  float scale = 1.0f;
+  if (flags & CHAIN_NORM_INPUT) {
+    float ss = 0.0f;   // same order as canonical_sumsq_lds: 16-byte units lane, lane+64, ...
+    for (u32 u = lane; u < (k_dim >> 2); u += 64u) {
+      ss = fmaf(x[4 * u], x[4 * u], ss); ss = fmaf(x[4 * u + 1], x[4 * u + 1], ss);
+      ss = fmaf(x[4 * u + 2], x[4 * u + 2], ss); ss = fmaf(x[4 * u + 3], x[4 * u + 3], ss);
+    }
+    scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(k_dim) + kChainNormEps);
+  }
   for (u32 row = block_id * waves + wave; row < n_dim; row += num_blocks * waves) {
     const uint8_t* rp = w + static_cast<size_t>(row) * nsb * SB;
     float acc = 0.0f;
@@ -119,23 +52,50 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
       }
     }
     acc = wave_sum(acc);
-    if (lane == 0) y[row] = acc;
+    if (lane == 0) y[row] = acc * scale;
   }
 }
 
 #define KQ_GEMV_KERNELS(fmtname, FMT)                                                                    \
   extern "C" __global__ void __launch_bounds__(512)                                                      \
       fmtname##_gemv_warp_reduce(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim) {     \
-    gemv_fast_body<FMT, 2>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x);                                \
+    extern __shared__ f32x4 lds4[];                                                                      \
+    __shared__ u32 s_flag;                                                                               \
+    const ChainEntry e = {FMT, k_dim, n_dim, 0u, w, x, y};                                               \
+    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                          \
+  }                                                                                                      \
+  extern "C" __global__ void __launch_bounds__(512)                                                      \
+      fmtname##_gemv_flags(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) {\
+    extern __shared__ f32x4 lds4[];                                                                      \
+    __shared__ u32 s_flag;                                                                               \
+    const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
+    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
-      fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim) {         \
-    gemv_generic_body<FMT, POLICY_GEMV>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x);                   \
+      fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
+    gemv_generic_body<FMT, POLICY_GEMV>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x, flags);            \
   }
 
 KQ_GEMV_KERNELS(q4k, FMT_Q4K)
 KQ_GEMV_KERNELS(q5k, FMT_Q5K)
 KQ_GEMV_KERNELS(q6k, FMT_Q6K)
+
+// The whole list in one cooperative launch (kquant_chain.hip.h).
+extern "C" __global__ void __launch_bounds__(512)
+kq_gemv_chain(const ChainEntry* entries, u32 count, u32* counters, u32* status, u32 spin_limit, u32 prefetch) {
+  chain_body<2>(entries, count, counters, status, spin_limit, prefetch);
+}
+
+// The list with decoupled weight streaming (kquant_stream.hip.h): one workgroup per CU.
+extern "C" __global__ void __launch_bounds__(512)
+kq_gemv_stream(const ChainEntry* entries, u32 count, u32* counters, u32* status, u32 spin_limit, u32 x_bytes_max,
+               u32 rows_max, u32 slabs_max) {
+  stream::stream_body(entries, count, counters, status, spin_limit, x_bytes_max, rows_max, slabs_max);
+}
+
+extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32 v) {
+  for (u32 i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = v;
+}
 
 // ------------------------------------------------------------------------------------------
 // Batched GEMM  C[m x n] = A[m x k] . dequant(W[n x k])^T,  c[row*n + col] (quantize.rs:568-574).
@@ -145,9 +105,12 @@ KQ_GEMV_KERNELS(q6k, FMT_Q6K)
 #define KQ_GEMM_KERNELS(fmtname, FMT)                                                                    \
   extern "C" __global__ void __launch_bounds__(512)                                                      \
       fmtname##_gemm_ggml(const float* a, const uint8_t* b_quant, float* c, u32 m, u32 n, u32 k) {       \
+    extern __shared__ f32x4 lds4[];                                                                      \
+    __shared__ u32 s_flag;                                                                               \
     for (u32 r = blockIdx.y; r < m; r += gridDim.y) {                                                    \
-      gemv_fast_body<FMT, 2>(c + static_cast<size_t>(r) * n, b_quant, a + static_cast<size_t>(r) * k,    \
-                             k, n, blockIdx.x, gridDim.x);                                               \
+      const ChainEntry e = {FMT, k, n, 0u, b_quant, a + static_cast<size_t>(r) * k,                      \
+                            c + static_cast<size_t>(r) * n};                                             \
+      chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                        \
       __syncthreads();                                                                                   \
     }                                                                                                    \
   }                                                                                                      \
@@ -155,7 +118,7 @@ KQ_GEMV_KERNELS(q6k, FMT_Q6K)
       fmtname##_gemm_generic(const float* a, const uint8_t* b_quant, float* c, u32 m, u32 n, u32 k) {    \
     for (u32 r = blockIdx.y; r < m; r += gridDim.y)                                                      \
       gemv_generic_body<FMT, POLICY_GEMV>(c + static_cast<size_t>(r) * n, b_quant,                       \
-                                          a + static_cast<size_t>(r) * k, k, n, blockIdx.x, gridDim.x);  \
+                                          a + static_cast<size_t>(r) * k, k, n, blockIdx.x, gridDim.x, 0u); \
   }
 
 KQ_GEMM_KERNELS(q4k, FMT_Q4K)

@@ -12,10 +12,13 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <cstdio>
 #include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 // ---- embedded code object -------------------------------------------------------------------
 #ifndef TRN_HSACO_PATH
@@ -45,12 +48,18 @@ enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2 };
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
+constexpr uint32_t kLdsScratch = 64;           // reduction scratch at the end of the fast kernels' LDS
+constexpr uint32_t kFlagNormInput = 1u, kFlagBarrierBefore = 2u, kFlagSameX = 4u;   // CHAIN_* of kquant_chain.hip.h
+// kquant_stream.hip.h: control block, ring (+16 mirror bytes), activations, partial sums, counters
+constexpr uint32_t kStreamCtlBytes = 256, kStreamRingBytes = 96 * 1024, kStreamLdsLimit = 160 * 1024 - 1024;
 
 struct DeviceKernels {
   bool loaded = false;
   hipModule_t module = nullptr;
   int cu_count = 0;
-  hipFunction_t gemv_fast[NFMT] = {}, gemv_generic[NFMT] = {};
+  hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
+  hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr;
+  int cooperative = 0;
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
@@ -60,6 +69,12 @@ std::mutex g_mutex;
 DeviceKernels g_dev[kMaxDevices];
 int g_tune_blocks_per_cu = 0;
 int g_tune_row_groups = 0;
+int g_tune_batch_mode = 0;   // 0: one launch per entry (default); 1: resident workgroups + barriers; 2: 1 + streaming producer
+int g_tune_chain_blocks_per_cu = 0;
+int g_tune_chain_waves = 0;
+int g_tune_chain_spin_limit = 0;
+int g_tune_chain_prefetch_off = 0;
+int g_tune_stream_consumers = 0;
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -89,6 +104,7 @@ hipError_t device_kernels(DeviceKernels** out) {
     for (int f = 0; f < NFMT; ++f) {
       const std::string p = kFmtName[f];
       if ((e = get_fn(m, &t.gemv_fast[f], p + "_gemv_warp_reduce")) != hipSuccess ||
+          (e = get_fn(m, &t.gemv_flags[f], p + "_gemv_flags")) != hipSuccess ||
           (e = get_fn(m, &t.gemv_generic[f], p + "_gemv_generic")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_fast[f], p + "_gemm_ggml")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_generic[f], p + "_gemm_generic")) != hipSuccess ||
@@ -98,7 +114,10 @@ hipError_t device_kernels(DeviceKernels** out) {
         return e;
       }
     }
-    if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess) {
+    if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
+        (e = get_fn(m, &t.chain, "kq_gemv_chain")) != hipSuccess ||
+        (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
+        (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
     }
@@ -107,6 +126,7 @@ hipError_t device_kernels(DeviceKernels** out) {
       return e;
     }
     if (t.cu_count <= 0) t.cu_count = 256;
+    (void)hipDeviceGetAttribute(&t.cooperative, hipDeviceAttributeCooperativeLaunch, dev);
     t.loaded = true;
     d = t;
   }
@@ -135,13 +155,13 @@ GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n) {
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
   // keep activations + partial sums within the LDS the kernel may ask for
   const uint64_t x_bytes = uint64_t(k) * 4u;
-  if (x_bytes + uint64_t(sw) * ug * 4u > kFastLdsLimit) return g;
-  const uint64_t max_rows = (kFastLdsLimit - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
+  if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return g;
+  const uint64_t max_rows = (kFastLdsLimit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
   rows = std::min<uint64_t>(rows, max_rows);
   g.grid = uint32_t((uint64_t(n) + rows - 1) / rows);
   // the kernel recomputes rows-per-block from the grid; it can only come out <= rows
   g.block = 64u * sw * groups;
-  g.lds = uint32_t(x_bytes + uint64_t(sw) * rows * 4u);
+  g.lds = uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch);
   g.fits = true;
   return g;
 }
@@ -155,7 +175,7 @@ bool gemv_fast_ok(Fmt f, uint64_t y, uint64_t w, uint64_t x) {
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
-                            uint32_t k, bool is_gemv) {
+                            uint32_t k, bool is_gemv, uint32_t flags = 0) {
   if (k % 256u != 0) return hipErrorInvalidValue;
   if (n == 0 || m == 0) return hipSuccess;
   if ((a == 0 && k != 0) || c == 0 || (w == 0 && k != 0)) return hipErrorInvalidValue;
@@ -164,14 +184,14 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   if (e != hipSuccess) return e;
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
-  void* gemv_args[] = {&c, &w, &a, &k, &n};
+  void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
   void* gemm_args[] = {&a, &w, &c, &m, &n, &k};
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
   if (k != 0 && gemv_fast_ok(f, c, w, a) && (is_gemv || (aligned(uint64_t(k) * 4u, 16) && aligned(uint64_t(n) * 4u, 4))))
     g = gemv_geometry(*d, k, n);
   if (g.fits) {
-    hipFunction_t fn = is_gemv ? d->gemv_fast[f] : d->gemm_fast[f];
+    hipFunction_t fn = is_gemv ? (flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
     return hipModuleLaunchKernel(fn, g.grid, is_gemv ? 1u : grid_y, 1, g.block, 1, 1, g.lds, stream, args, nullptr);
   }
   hipFunction_t fn = is_gemv ? d->gemv_generic[f] : d->gemm_generic[f];
@@ -196,6 +216,209 @@ hipError_t launch_dequant(Fmt f, hipStream_t stream, uint64_t out, uint64_t w, u
   }
   void* args[] = {&out, &w, &n_sb, &policy};
   return hipModuleLaunchKernel(d->dequant_generic[f], grid, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
+}
+
+// ---- the persistent executor behind trn_kquant_gemv_batch ---------------------------------------
+struct ChainEntryHost {  // ChainEntry of kquant_chain.hip.h
+  uint32_t fmt, k, n, flags;
+  uint64_t w, x, y;
+};
+static_assert(sizeof(ChainEntryHost) == 40, "ChainEntry layout");
+
+struct ChainWorkspace {
+  void* d_entries = nullptr;
+  size_t cap_entries = 0;
+  uint32_t* d_counters = nullptr;
+  size_t cap_counters = 0;
+  uint32_t* h_status = nullptr;  // pinned, device-visible: set by the kernel if a barrier wait gave up
+  uint32_t* d_status = nullptr;
+  std::vector<ChainEntryHost> last;
+  uint32_t grid = 0, block = 0, lds = 0, barriers = 0;
+};
+std::map<std::pair<int, hipStream_t>, ChainWorkspace> g_chain_ws;
+
+// words one barrier owns: top counter + one counter per group of 32 workgroups, 256 bytes apart
+// (chain_barrier_stride of kquant_chain.hip.h)
+uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u + (num_workgroups + 31u) / 32u); }
+
+bool ranges_overlap(uint64_t a, uint64_t alen, uint64_t b, uint64_t blen) { return a < b + blen && b < a + alen; }
+
+// Runs the list as one cooperative launch when every entry qualifies for the fast kernels.
+// *handled = false (and hipSuccess) means the caller should issue the entries one by one.
+hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t count, bool* handled) {
+  *handled = false;
+  if (g_tune_batch_mode == 0 || count < 2) return hipSuccess;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  if (!d->cooperative) return hipSuccess;
+  for (uint32_t i = 0; i < count; ++i) {
+    const trn_gemv_desc& g = descs[i];
+    if (g.n == 0 || g.k == 0 || !g.x || !g.w || !g.y) return hipSuccess;
+    if (!gemv_fast_ok(Fmt(g.fmt - 4), g.y, g.w, g.x)) return hipSuccess;
+  }
+  // entries: barrier where an entry touches what an entry of the current group wrote (or overwrites
+  // what one of them reads)
+  std::vector<ChainEntryHost> entries(count);
+  uint32_t barriers = 0;
+  size_t group_begin = 0;
+  for (uint32_t i = 0; i < count; ++i) {
+    const trn_gemv_desc& g = descs[i];
+    bool dep = false;
+    for (size_t j = group_begin; j < i && !dep; ++j) {
+      const trn_gemv_desc& p = descs[j];
+      dep = ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
+            ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
+    }
+    if (dep) {
+      ++barriers;
+      group_begin = i;
+    }
+    entries[i] = {g.fmt, g.k, g.n, g.flags | (dep ? kFlagBarrierBefore : 0u), g.w, g.x, g.y};
+  }
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  ChainWorkspace* ws;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    ws = &g_chain_ws[std::make_pair(dev, stream)];
+  }
+  if (!ws->h_status) {
+    if ((e = hipHostMalloc(reinterpret_cast<void**>(&ws->h_status), 64, hipHostMallocMapped)) != hipSuccess) return e;
+    ws->h_status[0] = 0;
+    if ((e = hipHostGetDevicePointer(reinterpret_cast<void**>(&ws->d_status), ws->h_status, 0)) != hipSuccess) return e;
+  }
+  if (ws->h_status[0] != 0) {  // an earlier list on this stream gave up at a wait: report it once
+    ws->h_status[0] = 0;
+    return hipErrorLaunchFailure;
+  }
+
+  // ---- streaming form: one workgroup per CU, a producer wave feeding an LDS ring -------------------
+  bool use_stream = g_tune_batch_mode == 2;
+  uint32_t consumers = g_tune_stream_consumers > 0 ? uint32_t(g_tune_stream_consumers) : 7u;
+  consumers = std::max(1u, std::min(consumers, 7u));
+  const uint32_t sgrid = uint32_t(d->cu_count);
+  uint32_t x_bytes_max = 0, rows_max = 1, slabs_max = 1;
+  for (uint32_t i = 0; i < count && use_stream; ++i) {
+    const trn_gemv_desc& g = descs[i];
+    const uint32_t nsb = g.k / 256u, slabs = (nsb + 15u) / 16u;
+    const uint64_t row_bytes = uint64_t(nsb) * kSbBytes[g.fmt - 4];
+    const uint64_t rows = (uint64_t(g.n) + sgrid - 1) / sgrid;
+    if (slabs > consumers || (uint64_t(g.n) * row_bytes) % 16u != 0 || rows * row_bytes >= (1ull << 31)) use_stream = false;
+    x_bytes_max = std::max<uint32_t>(x_bytes_max, g.k * 4u);
+    slabs_max = std::max(slabs_max, slabs);
+    if (slabs > 1) rows_max = std::max<uint32_t>(rows_max, uint32_t(rows));
+  }
+  uint32_t slds = kStreamCtlBytes + kStreamRingBytes + 16u + x_bytes_max + rows_max * slabs_max * 4u + rows_max * 4u;
+  if (slds > kStreamLdsLimit) use_stream = false;
+  if (use_stream) {
+    // entries that read the same vector (same length, same register layout) as their predecessor,
+    // with no barrier in between, keep the activations where they are
+    for (uint32_t i = 1; i < count; ++i) {
+      const bool q6a = descs[i].fmt == 6, q6b = descs[i - 1].fmt == 6;
+      if (!(entries[i].flags & kFlagBarrierBefore) && descs[i].x == descs[i - 1].x && descs[i].k == descs[i - 1].k && q6a == q6b)
+        entries[i].flags |= kFlagSameX;
+    }
+  }
+  auto upload = [&](uint32_t grid_for_counters) -> hipError_t {
+    const bool same = ws->last.size() == entries.size() &&
+                      std::memcmp(ws->last.data(), entries.data(), entries.size() * sizeof(ChainEntryHost)) == 0;
+    if (!same) {
+      hipError_t err = hipStreamSynchronize(stream);  // the device copy may still be read by a list in flight
+      if (err != hipSuccess) return err;
+      if (ws->cap_entries < entries.size()) {
+        if (ws->d_entries) (void)hipFree(ws->d_entries);
+        ws->d_entries = nullptr;
+        ws->cap_entries = 0;
+        if ((err = hipMalloc(&ws->d_entries, entries.size() * sizeof(ChainEntryHost))) != hipSuccess) return err;
+        ws->cap_entries = entries.size();
+      }
+      if ((err = hipMemcpy(ws->d_entries, entries.data(), entries.size() * sizeof(ChainEntryHost), hipMemcpyHostToDevice)) != hipSuccess)
+        return err;
+      ws->last = entries;
+    }
+    const size_t n_words = size_t(barriers + 1u) * chain_barrier_stride_host(grid_for_counters);
+    if (ws->cap_counters < n_words) {
+      hipError_t err = hipStreamSynchronize(stream);
+      if (err != hipSuccess) return err;
+      if (ws->d_counters) (void)hipFree(ws->d_counters);
+      ws->d_counters = nullptr;
+      ws->cap_counters = 0;
+      if ((err = hipMalloc(reinterpret_cast<void**>(&ws->d_counters), n_words * sizeof(uint32_t))) != hipSuccess) return err;
+      ws->cap_counters = n_words;
+    }
+    uint32_t n_counters = uint32_t(n_words), zero = 0u;
+    void* fill_args[] = {&ws->d_counters, &n_counters, &zero};
+    const uint32_t fill_grid = std::max(1u, std::min(64u, (n_counters + 255u) / 256u));
+    return hipModuleLaunchKernel(d->fill_u32, fill_grid, 1, 1, 256, 1, 1, 0, stream, fill_args, nullptr);
+  };
+  uint32_t spin_limit = g_tune_chain_spin_limit > 0 ? uint32_t(g_tune_chain_spin_limit) : 4000000u;
+  uint32_t cnt = count;
+  if (use_stream) {
+    if ((e = upload(sgrid)) != hipSuccess) return e;
+    void* args[] = {&ws->d_entries, &cnt, &ws->d_counters, &ws->d_status, &spin_limit, &x_bytes_max, &rows_max, &slabs_max};
+    e = hipModuleLaunchCooperativeKernel(d->stream, sgrid, 1, 1, 64u * (1u + consumers), 1, 1, slds, stream, args);
+    if (e == hipSuccess) {
+      ws->grid = sgrid; ws->block = 64u * (1u + consumers); ws->lds = slds; ws->barriers = barriers;
+      *handled = true;
+      return hipSuccess;
+    }
+    (void)hipGetLastError();   // not launchable in this form here: try the plain resident form below
+    for (auto& en : entries) en.flags &= ~kFlagSameX;
+  } else {
+    for (auto& en : entries) en.flags &= ~kFlagSameX;
+  }
+
+  // wave count per workgroup: the one that leaves the fewest waves idle, weighted by bytes
+  uint32_t waves = uint32_t(g_tune_chain_waves);
+  if (waves == 0) {
+    double best = -1.0;
+    for (uint32_t cand : {6u, 8u, 4u}) {
+      double useful = 0.0, total = 0.0;
+      for (uint32_t i = 0; i < count; ++i) {
+        const uint32_t slabs = (descs[i].k / 256u + 15u) / 16u, sw = std::min(slabs, cand);
+        const double bytes = double(descs[i].n) * descs[i].k;
+        useful += bytes * double(sw * (cand / sw)) / cand;
+        total += bytes;
+      }
+      if (useful / total > best + 1e-9) { best = useful / total; waves = cand; }
+    }
+  }
+  waves = std::max(1u, std::min(waves, 8u));
+  const uint32_t block = 64u * waves;
+  auto lds_for = [&](uint32_t grid) {
+    uint32_t lds = 0;
+    for (uint32_t i = 0; i < count; ++i) {
+      const uint32_t slabs = (descs[i].k / 256u + 15u) / 16u, sw = std::min(slabs, waves);
+      uint64_t rows = (uint64_t(descs[i].n) + grid - 1) / grid;
+      rows = (rows + kGemvRowsPerBatch - 1) / kGemvRowsPerBatch * kGemvRowsPerBatch;
+      const uint64_t need = uint64_t(descs[i].k) * 4u + uint64_t(sw) * rows * 4u + kLdsScratch;
+      if (need > kFastLdsLimit) return 0u;
+      lds = std::max<uint32_t>(lds, uint32_t(need));
+    }
+    return lds;
+  };
+  uint32_t lds = lds_for(uint32_t(d->cu_count));
+  if (lds == 0) return hipSuccess;
+  int per_cu = 0;
+  if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, d->chain, int(block), lds) != hipSuccess || per_cu < 1)
+    return hipSuccess;
+  if (g_tune_chain_blocks_per_cu > 0) per_cu = std::min(per_cu, g_tune_chain_blocks_per_cu);
+  per_cu = std::min(per_cu, 2);  // barrier cost grows with the number of workgroups
+  const uint32_t grid = uint32_t(d->cu_count) * uint32_t(per_cu);
+  lds = lds_for(grid);
+
+  if ((e = upload(grid)) != hipSuccess) return e;
+  ws->grid = grid; ws->block = block; ws->lds = lds; ws->barriers = barriers;
+  uint32_t prefetch = g_tune_chain_prefetch_off ? 0u : 1u;
+  void* args[] = {&ws->d_entries, &cnt, &ws->d_counters, &ws->d_status, &spin_limit, &prefetch};
+  e = hipModuleLaunchCooperativeKernel(d->chain, grid, 1, 1, block, 1, 1, lds, stream, args);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return hipSuccess;  // not launchable as one resident grid here: the caller issues the entries one by one
+  }
+  *handled = true;
+  return hipSuccess;
 }
 
 }  // namespace
@@ -243,7 +466,17 @@ trn_status trn_device_get(trn_device* device, int ordinal) {
 
 trn_status trn_device_get_name(char* name, int len, trn_device device) {
   if (!name || len <= 0) return TRN_ERROR_INVALID_VALUE;
-  return st(hipDeviceGetName(name, len, static_cast<hipDevice_t>(device)));
+  name[0] = 0;
+  hipError_t e = hipDeviceGetName(name, len, static_cast<hipDevice_t>(device));
+  if (e != hipSuccess) return st(e);
+  if (name[0] == 0) {   // some driver stacks leave the marketing name empty: fall back to the ISA name
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, static_cast<int>(device));
+    if (e != hipSuccess) return st(e);
+    const char* src = prop.name[0] ? prop.name : prop.gcnArchName;
+    snprintf(name, static_cast<size_t>(len), "%s", src);
+  }
+  return TRN_SUCCESS;
 }
 
 trn_status trn_device_total_mem(size_t* bytes, trn_device device) {
@@ -466,10 +699,15 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   if (count == 0) return TRN_SUCCESS;
   if (!descs) return TRN_ERROR_INVALID_VALUE;
   for (uint32_t i = 0; i < count; ++i)  // validate the whole list before anything is launched
-    if (descs[i].fmt < 4 || descs[i].fmt > 6 || descs[i].reserved != 0 || descs[i].k % 256u != 0) return TRN_ERROR_INVALID_VALUE;
+    if (descs[i].fmt < 4 || descs[i].fmt > 6 || (descs[i].flags & ~TRN_GEMV_NORM_INPUT) != 0 || descs[i].k % 256u != 0)
+      return TRN_ERROR_INVALID_VALUE;
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  bool handled = false;
+  hipError_t e = launch_chain(stream, descs, count, &handled);
+  if (handled || e != hipSuccess) return st(e);
   for (uint32_t i = 0; i < count; ++i) {
     const trn_gemv_desc& d = descs[i];
-    hipError_t e = launch_gemm_like(Fmt(d.fmt - 4), static_cast<hipStream_t>(s), d.x, d.w, d.y, 1, d.n, d.k, true);
+    e = launch_gemm_like(Fmt(d.fmt - 4), stream, d.x, d.w, d.y, 1, d.n, d.k, true, d.flags);
     if (e != hipSuccess) return st(e);
   }
   return TRN_SUCCESS;
@@ -544,6 +782,12 @@ trn_status trn_set_tuning(const char* key, int value) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!std::strcmp(key, "gemv_blocks_per_cu")) { g_tune_blocks_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_row_groups")) { g_tune_row_groups = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "batch_mode")) { g_tune_batch_mode = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "chain_blocks_per_cu")) { g_tune_chain_blocks_per_cu = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "chain_waves")) { g_tune_chain_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "chain_spin_limit")) { g_tune_chain_spin_limit = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 

@@ -212,8 +212,10 @@ class GemvBatch:
         self._entries = []
         self._array = None
 
-    def add(self, fmt: str, k: int, n: int, y, w, x) -> "GemvBatch":
-        self._entries.append(_ffi.GemvDesc(self._FMT[fmt], int(k), int(n), 0, _ptr(y), _ptr(w), _ptr(x)))
+    NORM_INPUT = 1  # the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x
+
+    def add(self, fmt: str, k: int, n: int, y, w, x, flags: int = 0) -> "GemvBatch":
+        self._entries.append(_ffi.GemvDesc(self._FMT[fmt], int(k), int(n), int(flags), _ptr(y), _ptr(w), _ptr(x)))
         self._array = None
         return self
 
