@@ -124,7 +124,9 @@ TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
  * roadmap.yaml:359-368).  Entry i computes y = dequant(W) x exactly as the typed launcher of its
  * format would; a later entry may read what an earlier one wrote (the library finds those
  * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
- * By default the list is issued as one launch per entry.  With trn_set_tuning("batch_mode", 1 or 2),
+ * By default the list is issued as one launch per entry, except that up to four neighbouring entries
+ * with the same k that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share
+ * one launch.  With trn_set_tuning("batch_mode", 1 or 2),
  * and when every entry meets the fast kernels' alignment (x 16 B, W 16 B / 2 B for Q6_K), the list
  * runs as ONE cooperative launch of resident workgroups with device-side barriers at the
  * dependencies.  That form keeps, per (device, stream), a small device buffer with the list and its
@@ -170,7 +172,8 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * launch per entry (default), 1 one cooperative launch of resident workgroups with device-side
  * barriers, 2 as 1 with a producer wave per CU streaming the weights through an LDS ring.
  * "chain_blocks_per_cu", "chain_waves", "chain_prefetch_off", "stream_consumers": geometry of modes 1/2.
- * "chain_spin_limit": polls a device-side barrier wait may take before it gives up. */
+ * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
+ * "group_off": 1 = in mode 0 never fuse neighbouring independent entries of a list into one launch. */
 TRN_API trn_status trn_set_tuning(const char* key, int value);
 
 #ifdef __cplusplus

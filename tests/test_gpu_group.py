@@ -1,0 +1,73 @@
+"""GPU parity: neighbouring independent entries of a GEMV list share one launch; the results must have the
+same bits as with one launch per entry (fusing switched off), and match the fp64 oracle."""
+import numpy as np
+import pytest
+
+import trueno_amd as t
+from oracle import kquant as kq
+from trueno_amd import _ffi
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def _tune(key, value):
+    assert _ffi.lib().trn_set_tuning(key.encode(), int(value)) == 0
+
+
+def _run(gpu, specs, x_len, group_off):
+    ctx, stream = gpu
+    host = {"x": kq.gen_x(1, x_len)}
+    bufs = {"x": t.GpuBuffer.from_host(ctx, host["x"])}
+    mats, keep, batch = [], [], t.GemvBatch()
+    for i, (fmt, n, k, src, dst, flags) in enumerate(specs):
+        if dst not in bufs:
+            bufs[dst] = t.GpuBuffer.from_host(ctx, np.full(n, np.nan, np.float32))
+        m = kq.gen_matrix(fmt, 900 + i, n, k)
+        mats.append(m)
+        w = t.GpuBuffer.from_host(ctx, m)
+        keep.append(w)            # the list holds raw pointers: the buffers must outlive the launch
+        batch.add(fmt, k, n, bufs[dst], w, bufs[src], flags)
+    _tune("group_off", group_off)
+    try:
+        batch.launch(stream)
+        stream.synchronize()
+    finally:
+        _tune("group_off", 0)
+    return {k: v.copy_to_host() for k, v in bufs.items()}, mats
+
+
+CASES = {
+    # q, k, v share x; o depends on q; gate, up share o's output; down depends on gate
+    "layer": ([("q4k", 1024, 1024, "x", "q", 1), ("q4k", 1024, 1024, "x", "k", 1), ("q4k", 1024, 1024, "x", "v", 1),
+               ("q4k", 1024, 1024, "q", "o", 1), ("q4k", 2816, 1024, "o", "g", 1), ("q4k", 2816, 1024, "o", "u", 1),
+               ("q6k", 1024, 2816, "g", "d", 1)], 1024),
+    # mixed formats and ragged row counts in one group; five independent entries (a group holds four)
+    "mixed": ([("q4k", 37, 512, "x", "a", 0), ("q5k", 513, 512, "x", "b", 1), ("q6k", 300, 512, "x", "c", 1),
+               ("q4k", 64, 512, "x", "d", 0), ("q5k", 129, 512, "x", "e", 1)], 512),
+    # different k next to each other must not be fused; write-after-read must not be fused
+    "no_fuse": ([("q4k", 512, 512, "x", "a", 1), ("q4k", 256, 768, "x", "b", 1), ("q4k", 512, 512, "a", "x2", 0),
+                 ("q4k", 512, 512, "x2", "a", 0)], 768),
+}
+
+
+@pytest.mark.parametrize("case", sorted(CASES))
+def test_grouped_equals_separate(gpu, case):
+    specs, x_len = CASES[case]
+    sep, _ = _run(gpu, specs, x_len, 1)
+    got, mats = _run(gpu, specs, x_len, 0)
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), (case, name)
+    # the chain against fp64, entry by entry, each on the input the GPU actually used
+    final = {}
+    for (fmt, n, k, src, dst, flags), m in zip(specs, mats):
+        final[dst] = (fmt, n, k, src, flags, m)
+    for dst, (fmt, n, k, src, flags, m) in final.items():
+        if case == "no_fuse" and dst in ("a", "x2"):
+            continue            # overwritten or re-read later in the list
+        x = got[src][:k].astype(np.float64)
+        ref = kq.dequant_matrix(fmt, m, n, k).astype(np.float64) @ x
+        if flags:
+            ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
+        assert kq.rel_l2(got[dst], ref) <= TOL, (case, dst)

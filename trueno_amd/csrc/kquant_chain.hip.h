@@ -50,7 +50,15 @@ constexpr float kChainNormEps = 1e-6f;
 template <class Q>
 __device__ __forceinline__ float canonical_sumsq_lds(const f32x4* lds4, u32 units, u32 lane) {
   float ss = 0.0f;
-  for (u32 u = lane; u < units; u += 64u) {
+  u32 u = lane;
+  for (; u + 192u < units; u += 256u) {      // four reads in flight; the additions keep their order
+    const f32x4 v0 = lds4[Q::swz(u)], v1 = lds4[Q::swz(u + 64u)], v2 = lds4[Q::swz(u + 128u)], v3 = lds4[Q::swz(u + 192u)];
+    ss = fmaf(v0.x, v0.x, ss); ss = fmaf(v0.y, v0.y, ss); ss = fmaf(v0.z, v0.z, ss); ss = fmaf(v0.w, v0.w, ss);
+    ss = fmaf(v1.x, v1.x, ss); ss = fmaf(v1.y, v1.y, ss); ss = fmaf(v1.z, v1.z, ss); ss = fmaf(v1.w, v1.w, ss);
+    ss = fmaf(v2.x, v2.x, ss); ss = fmaf(v2.y, v2.y, ss); ss = fmaf(v2.z, v2.z, ss); ss = fmaf(v2.w, v2.w, ss);
+    ss = fmaf(v3.x, v3.x, ss); ss = fmaf(v3.y, v3.y, ss); ss = fmaf(v3.z, v3.z, ss); ss = fmaf(v3.w, v3.w, ss);
+  }
+  for (; u < units; u += 64u) {
     const f32x4 v = lds4[Q::swz(u)];
     ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
   }
@@ -129,16 +137,17 @@ __device__ __forceinline__ u32 chain_prefetch(const ChainEntry& e) {
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
 template <int FMT, int U, bool COHERENT = false>
 __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
-                                           f32x4* lds4, u32* s_flag, const ChainEntry* next = nullptr, u32* sink = nullptr) {
+                                           f32x4* lds4, u32* s_flag, const ChainEntry* next, u32* sink,
+                                           u32 block_id, u32 num_blocks) {
   using Q = Quarter<FMT>;
   const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;
   const u32 sw_count = slabs < waves ? slabs : waves;
   const u32 groups = waves / sw_count;
-  u32 rows_per_block = (n_dim + gridDim.x - 1) / gridDim.x;
+  u32 rows_per_block = (n_dim + num_blocks - 1) / num_blocks;
   rows_per_block = ((rows_per_block + U - 1) / U) * U;
-  const u32 row0 = blockIdx.x * rows_per_block;
+  const u32 row0 = block_id * rows_per_block;
   const bool has_rows = row0 < n_dim && nsb != 0;
   const u32 batches = has_rows ? rows_per_block / U : 0u;
   const u32 sw = wave % sw_count, grp = wave / sw_count;
@@ -251,9 +260,9 @@ __device__ __forceinline__ void chain_body(const ChainEntry* __restrict__ entrie
     u32* wait_counter = (e.flags & CHAIN_BARRIER_BEFORE) ? counters + bar * chain_barrier_stride(gridDim.x) : nullptr;
     bool ok = true;
     const ChainEntry* next = (prefetch && i + 1 < count) ? entries + i + 1 : nullptr;
-    if (e.fmt == FMT_Q4K) ok = chain_step<FMT_Q4K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
-    else if (e.fmt == FMT_Q5K) ok = chain_step<FMT_Q5K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
-    else if (e.fmt == FMT_Q6K) ok = chain_step<FMT_Q6K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1);
+    if (e.fmt == FMT_Q4K) ok = chain_step<FMT_Q4K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
+    else if (e.fmt == FMT_Q5K) ok = chain_step<FMT_Q5K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
+    else if (e.fmt == FMT_Q6K) ok = chain_step<FMT_Q6K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
     if (!ok) return;
     if (wait_counter) ++bar;
     const bool arrive = i + 1 < count && (entries[i + 1].flags & CHAIN_BARRIER_BEFORE) != 0u;

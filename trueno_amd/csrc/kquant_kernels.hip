@@ -62,14 +62,14 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, 0u, w, x, y};                                               \
-    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                          \
+    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(512)                                                      \
       fmtname##_gemv_flags(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) {\
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
-    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                          \
+    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
@@ -79,6 +79,26 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
 KQ_GEMV_KERNELS(q4k, FMT_Q4K)
 KQ_GEMV_KERNELS(q5k, FMT_Q5K)
 KQ_GEMV_KERNELS(q6k, FMT_Q6K)
+
+// Up to four GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
+// up) in one launch: consecutive runs of workgroups belong to consecutive entries.  Each entry is computed
+// exactly as its own launch would compute it.
+struct GemvGroup {
+  ChainEntry e[4];
+  u32 first[5];      // first[i] .. first[i+1]-1 are the workgroups of entry i
+  u32 count;
+};
+extern "C" __global__ void __launch_bounds__(512) kq_gemv_group(const GemvGroup g) {
+  extern __shared__ f32x4 lds4[];
+  __shared__ u32 s_flag;
+  u32 i = 0;
+  while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) ++i;
+  const ChainEntry e = g.e[i];
+  const u32 block_id = blockIdx.x - g.first[i], num_blocks = g.first[i + 1] - g.first[i];
+  if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, block_id, num_blocks);
+  else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, block_id, num_blocks);
+  else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, block_id, num_blocks);
+}
 
 // The whole list in one cooperative launch (kquant_chain.hip.h).
 extern "C" __global__ void __launch_bounds__(512)
@@ -110,7 +130,7 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
     for (u32 r = blockIdx.y; r < m; r += gridDim.y) {                                                    \
       const ChainEntry e = {FMT, k, n, 0u, b_quant, a + static_cast<size_t>(r) * k,                      \
                             c + static_cast<size_t>(r) * n};                                             \
-      chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag);                                        \
+      chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                        \
       __syncthreads();                                                                                   \
     }                                                                                                    \
   }                                                                                                      \

@@ -58,7 +58,7 @@ struct DeviceKernels {
   hipModule_t module = nullptr;
   int cu_count = 0;
   hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
-  hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr;
+  hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr;
   int cooperative = 0;
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
@@ -75,6 +75,7 @@ int g_tune_chain_waves = 0;
 int g_tune_chain_spin_limit = 0;
 int g_tune_chain_prefetch_off = 0;
 int g_tune_stream_consumers = 0;
+int g_tune_group_off = 0;   // 1: never fuse independent GEMVs of a list into one launch
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -117,6 +118,7 @@ hipError_t device_kernels(DeviceKernels** out) {
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
         (e = get_fn(m, &t.chain, "kq_gemv_chain")) != hipSuccess ||
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
+        (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -141,17 +143,19 @@ struct GemvGeometry {
   bool fits = false;
 };
 
-GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n) {
+GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint64_t n_for_rows = 0) {
   GemvGeometry g;
   const uint32_t nsb = k / 256u;
   const uint32_t slabs = (nsb + 15u) / 16u;
   const uint32_t sw = std::min<uint32_t>(slabs, 8u);
-  uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : std::max<uint32_t>(1u, 4u / sw);
+  // Measured on MI355X: one slab (k <= 4096) runs best as 4 workgroups of 4 waves per CU; with several
+  // slabs every workgroup stages the whole (large) activation vector, so one big workgroup per CU wins.
+  uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : 8u / sw);
   groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
   const uint32_t ug = kGemvRowsPerBatch * groups;
-  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : 4u;
+  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : (sw == 1 ? 4u : 1u);
   const uint64_t target_blocks = uint64_t(d.cu_count) * per_cu;
-  uint64_t rows = (uint64_t(n) + target_blocks - 1) / target_blocks;
+  uint64_t rows = (std::max<uint64_t>(n, n_for_rows) + target_blocks - 1) / target_blocks;
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
   // keep activations + partial sums within the LDS the kernel may ask for
   const uint64_t x_bytes = uint64_t(k) * 4u;
@@ -695,6 +699,41 @@ trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
   return st(launch_gemm_like(Q6K, static_cast<hipStream_t>(s), a, b, c, m, n, k, false));
 }
 
+namespace {
+struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip
+  ChainEntryHost e[4];
+  uint32_t first[5];
+  uint32_t count;
+};
+static_assert(sizeof(GemvGroupHost) == 4 * 40 + 5 * 4 + 4, "GemvGroup layout");
+
+bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) {
+  return ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
+         ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
+}
+
+// Entries first .. first+len-1 of a list (len in 2..4, same k, mutually independent, all meeting the fast
+// kernels' preconditions) as ONE launch.
+hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gemv_desc* descs, uint32_t len) {
+  uint64_t total_n = 0;
+  for (uint32_t i = 0; i < len; ++i) total_n += descs[i].n;
+  GemvGroupHost g{};
+  uint32_t block = 0, lds = 0;
+  g.first[0] = 0;
+  for (uint32_t i = 0; i < len; ++i) {
+    const GemvGeometry geo = gemv_geometry(*d, descs[i].k, descs[i].n, total_n);
+    if (!geo.fits) return hipErrorInvalidValue;
+    block = geo.block;
+    lds = std::max(lds, geo.lds);
+    g.e[i] = {descs[i].fmt, descs[i].k, descs[i].n, descs[i].flags, descs[i].w, descs[i].x, descs[i].y};
+    g.first[i + 1] = g.first[i] + geo.grid;
+  }
+  g.count = len;
+  void* args[] = {&g};
+  return hipModuleLaunchKernel(d->gemv_group, g.first[len], 1, 1, block, 1, 1, lds, stream, args, nullptr);
+}
+}  // namespace
+
 trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {
   if (count == 0) return TRN_SUCCESS;
   if (!descs) return TRN_ERROR_INVALID_VALUE;
@@ -705,10 +744,32 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   bool handled = false;
   hipError_t e = launch_chain(stream, descs, count, &handled);
   if (handled || e != hipSuccess) return st(e);
-  for (uint32_t i = 0; i < count; ++i) {
-    const trn_gemv_desc& d = descs[i];
-    e = launch_gemm_like(Fmt(d.fmt - 4), stream, d.x, d.w, d.y, 1, d.n, d.k, true, d.flags);
+  DeviceKernels* dk = nullptr;
+  if ((e = device_kernels(&dk)) != hipSuccess) return st(e);
+  auto groupable = [&](const trn_gemv_desc& d) {
+    return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
+           gemv_geometry(*dk, d.k, d.n).fits;
+  };
+  for (uint32_t i = 0; i < count;) {
+    // longest run (up to 4) of entries with the same k that do not touch one another's vectors
+    uint32_t len = 1;
+    if (!g_tune_group_off && groupable(descs[i])) {
+      while (len < 4 && i + len < count) {
+        const trn_gemv_desc& c = descs[i + len];
+        bool ok = c.k == descs[i].k && groupable(c);
+        for (uint32_t j = i; j < i + len && ok; ++j) ok = !gemv_depends(c, descs[j]) && !gemv_depends(descs[j], c);
+        if (!ok) break;
+        ++len;
+      }
+    }
+    if (len >= 2) {
+      e = launch_gemv_group(dk, stream, descs + i, len);
+    } else {
+      const trn_gemv_desc& d = descs[i];
+      e = launch_gemm_like(Fmt(d.fmt - 4), stream, d.x, d.w, d.y, 1, d.n, d.k, true, d.flags);
+    }
     if (e != hipSuccess) return st(e);
+    i += len;
   }
   return TRN_SUCCESS;
 }
@@ -788,6 +849,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "chain_spin_limit")) { g_tune_chain_spin_limit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
