@@ -64,3 +64,77 @@ def test_gemm_edge_cases(gpu):
     assert np.all(c.copy_to_host() == 3.0)
     with pytest.raises(t.GpuError):
         t.QuantizeKernel.ggml(1, 1, 300).launch(stream, a, w, c)  # k % 256 != 0
+
+
+def _tune(key, value):
+    from trueno_amd import _ffi
+    assert _ffi.lib().trn_set_tuning(key.encode(), int(value)) == 0
+
+
+@pytest.mark.parametrize("m", (2, 9, 13, 33))
+@pytest.mark.parametrize("n,k", [(100, 512), (1000, 2304)])
+def test_q4k_gemm_matrix_core_form_ragged(gpu, n, k, m):
+    """Token counts that do not fill a tile of 8, row counts that do not fill a tile of 32."""
+    buf, a = kq.gen_matrix("q4k", 50 + m, n, k), kq.gen_x(60 + m, m, k)
+    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64("q4k", buf, a, n, k)) <= TOL
+
+
+def test_q4k_gemm_geometry_does_not_change_the_result(gpu):
+    n, k, m = 777, 2048, 24
+    buf, a = kq.gen_matrix("q4k", 91, n, k), kq.gen_x(92, m, k)
+    c64 = _c64("q4k", buf, a, n, k)
+    outs = {}
+    try:
+        for tiles in (1, 2):
+            for parts in (1, 2):
+                _tune("gemm_tiles_per_wave", tiles)
+                _tune("gemm_k_parts", parts)
+                outs[(tiles, parts)] = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+                assert kq.rel_l2(outs[(tiles, parts)], c64) <= TOL
+                again = gpu_gemm(gpu, "q4k", buf, a, m, n, k)      # two K parts are added in either order: same bits
+                assert np.array_equal(again.view(np.uint32), outs[(tiles, parts)].view(np.uint32))
+    finally:
+        _tune("gemm_tiles_per_wave", 0)
+        _tune("gemm_k_parts", 0)
+    for parts in (1, 2):
+        assert np.array_equal(outs[(1, parts)].view(np.uint32), outs[(2, parts)].view(np.uint32))
+    try:
+        _tune("gemm_mfma_off", 1)
+        valu = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    finally:
+        _tune("gemm_mfma_off", 0)
+    assert kq.rel_l2(valu, c64) <= TOL
+
+
+def test_q4k_gemm_no_worse_than_reference_order_f32(gpu):
+    """Per token, the error against fp64 stays within the slack of an f32 evaluation in the reference's
+    summation order (quantize.rs:1412-1518)."""
+    n, k, m = 512, 4096, 16
+    buf, a = kq.gen_matrix("q4k", 93, n, k), kq.gen_x(94, m, k)
+    w = kq.dequant_matrix("q4k", buf, n, k)
+    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    c64 = kq.gemm_fp64(a, w)
+    ref = np.stack([kq.gemv_ref_order_fp32(w, a[i]) for i in range(m)])
+    err_ref, err_ours = kq.rel_l2(ref, c64), kq.rel_l2(c, c64)
+    print(f"q4k gemm {m}x{n}x{k}: ours {err_ours:.3e} vs reference-order f32 {err_ref:.3e}")
+    assert err_ours <= 1.5 * err_ref + 1e-9
+
+
+def test_q4k_gemm_special_values(gpu):
+    """An all-zero token, a huge and a tiny token, and a token with an infinity (its outputs are not finite,
+    the other tokens are untouched)."""
+    n, k, m = 64, 512, 5
+    buf = kq.gen_matrix("q4k", 95, n, k)
+    a = kq.gen_x(96, m, k)
+    a[1] = 0.0
+    a[2] *= 1e30
+    a[3] *= 1e-30
+    a[4, 17] = np.inf
+    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    w = kq.dequant_matrix("q4k", buf, n, k)
+    c64 = kq.gemm_fp64(a[:4], w)
+    assert np.all(c[1] == 0.0)
+    for i in (0, 2, 3):
+        assert kq.rel_l2(c[i], c64[i]) <= TOL
+    assert not np.any(np.isfinite(c[4]))

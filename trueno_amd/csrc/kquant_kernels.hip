@@ -10,6 +10,7 @@
 // multiple of 64.
 #include "kquant_chain.hip.h"
 #include "kquant_stream.hip.h"
+#include "kquant_gemm_mfma.hip.h"
 
 // The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
 // activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
@@ -144,6 +145,20 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
 KQ_GEMM_KERNELS(q4k, FMT_Q4K)
 KQ_GEMM_KERNELS(q5k, FMT_Q5K)
 KQ_GEMM_KERNELS(q6k, FMT_Q6K)
+
+// Matrix-core form of the Q4_K GEMM for m >= 2 (kquant_gemm_mfma.hip.h): digit planes of A, then the product.
+extern "C" __global__ void __launch_bounds__(256)
+kq_gemm_planes(const float* a, uint8_t* planes, float* meta, float* c, u32 m, u32 n, u32 k, u32 clear_c) {
+  gemm_mfma::planes_body(a, planes, meta, c, m, n, k, clear_c);
+}
+extern "C" __global__ void __launch_bounds__(256)
+q4k_gemm_mfma_t1(const uint8_t* planes, const float* meta, const uint8_t* w, float* c, u32 m, u32 n, u32 k) {
+  gemm_mfma::q4k_body<1>(planes, meta, w, c, m, n, k);
+}
+extern "C" __global__ void __launch_bounds__(256)
+q4k_gemm_mfma_t2(const uint8_t* planes, const float* meta, const uint8_t* w, float* c, u32 m, u32 n, u32 k) {
+  gemm_mfma::q4k_body<2>(planes, meta, w, c, m, n, k);
+}
 
 // ------------------------------------------------------------------------------------------
 // Dequantise to f32 (test surface): out[sb*256 + i] = w_i.  The fast form shares load/unpack

@@ -63,6 +63,7 @@ struct DeviceKernels {
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
+  hipFunction_t gemm_planes = nullptr, gemm_mfma[2] = {};
 };
 
 std::mutex g_mutex;
@@ -75,7 +76,11 @@ int g_tune_chain_waves = 0;
 int g_tune_chain_spin_limit = 0;
 int g_tune_chain_prefetch_off = 0;
 int g_tune_stream_consumers = 0;
-int g_tune_group_off = 0;   // 1: never fuse independent GEMVs of a list into one launch
+int g_tune_group_off = 0;
+int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
+int g_tune_gemm_tiles = 0;      // token tiles (of 8) per wave in the matrix-core GEMM: 1 or 2
+int g_tune_gemm_ksplit = 0;     // parts of K per row tile: 1 or 2
+int g_tune_gemm_waves = 0;      // waves per workgroup of the matrix-core GEMM: 1..4   // 1: never fuse independent GEMVs of a list into one launch
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -119,6 +124,9 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.chain, "kq_gemv_chain")) != hipSuccess ||
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_planes, "kq_gemm_planes")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_mfma[0], "q4k_gemm_mfma_t1")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_mfma[1], "q4k_gemm_mfma_t2")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -178,6 +186,53 @@ bool gemv_fast_ok(Fmt f, uint64_t y, uint64_t w, uint64_t x) {
   return aligned(x, 16) && aligned(y, 4) && aligned(w, f == Q6K ? 2 : 16);
 }
 
+// Digit planes of A for the matrix-core GEMM: one buffer per (device, stream), grown on demand and kept.
+struct GemmWorkspace {
+  void* planes = nullptr;
+  size_t cap = 0;
+};
+std::map<std::pair<int, hipStream_t>, GemmWorkspace> g_gemm_ws;
+
+hipError_t launch_q4k_gemm_mfma(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
+                                uint32_t n, uint32_t k) {
+  const uint32_t nsb = k / 256u, tiles = (m + 7u) / 8u;
+  const size_t planes_bytes = size_t(tiles) * nsb * 8192u, meta_bytes = size_t(tiles) * nsb * 72u * 4u;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  GemmWorkspace* ws;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    ws = &g_gemm_ws[std::make_pair(dev, stream)];
+  }
+  if (ws->cap < planes_bytes + meta_bytes) {
+    if (ws->planes) {
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;   // a GEMM in flight may still read it
+      (void)hipFree(ws->planes);
+      ws->planes = nullptr;
+      ws->cap = 0;
+    }
+    if ((e = hipMalloc(&ws->planes, planes_bytes + meta_bytes)) != hipSuccess) return e;
+    ws->cap = planes_bytes + meta_bytes;
+  }
+  uint64_t planes = reinterpret_cast<uint64_t>(ws->planes), meta = planes + planes_bytes;
+  uint32_t t = g_tune_gemm_tiles > 0 ? uint32_t(g_tune_gemm_tiles) : 1u;   // measured: two tiles per wave never pay
+  t = std::min(std::max(t, 1u), 2u);
+  const uint32_t gx = (n + 31u) / 32u, gy = (tiles + t - 1u) / t;
+  uint32_t ksplit = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : (uint64_t(gx) * gy < uint64_t(d->cu_count) * 8u ? 2u : 1u);
+  ksplit = std::min(std::min(std::max(ksplit, 1u), 2u), nsb);
+  uint32_t clear_c = ksplit > 1 ? 1u : 0u;
+  void* pargs[] = {&a, &planes, &meta, &c, &m, &n, &k, &clear_c};
+  const uint64_t items = uint64_t(tiles) * 8u * nsb;
+  const uint32_t pgrid = uint32_t(std::min<uint64_t>((items + 3) / 4, uint64_t(d->cu_count) * 16u));
+  if ((e = hipModuleLaunchKernel(d->gemm_planes, pgrid, 1, 1, 256, 1, 1, 0, stream, pargs, nullptr)) != hipSuccess) return e;
+  void* margs[] = {&planes, &meta, &w, &c, &m, &n, &k};
+  // waves of a workgroup share a part of K: as many as leave each at least two super-blocks, four at most
+  uint32_t waves = g_tune_gemm_waves > 0 ? uint32_t(g_tune_gemm_waves) : 4u;
+  waves = std::max(1u, std::min(std::min(waves, 4u), std::max(1u, nsb / ksplit / 2u)));
+  return hipModuleLaunchKernel(d->gemm_mfma[t - 1], gx, gy, ksplit, 64 * waves, 1, 1, 0, stream, margs, nullptr);
+}
+
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
                             uint32_t k, bool is_gemv, uint32_t flags = 0) {
   if (k % 256u != 0) return hipErrorInvalidValue;
@@ -186,6 +241,9 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
+  if (!is_gemv && f == Q4K && m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
+      (n + 31u) / 32u <= 65535u * 32u && (m + 7u) / 8u <= 65535u)
+    return launch_q4k_gemm_mfma(d, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
@@ -850,6 +908,10 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_tiles_per_wave")) { g_tune_gemm_tiles = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
