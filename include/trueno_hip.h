@@ -98,7 +98,8 @@ TRN_API trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigne
  * reference does CudaModule::from_ptx(&ctx, &kernel.emit_ptx()) (driver/module.rs:62-79,
  * kernels/mod.rs:65-67).  It exports, with the reference's parameter lists:
  *   q4k_gemv_warp_reduce  q5k_gemv_warp_reduce  q6k_gemv_warp_reduce   (y, w, x, k_dim, n_dim)
- *   q4k_gemm_ggml         q5k_gemm_ggml         q6k_gemm_ggml          (a, b_quant, c, m, n, k) */
+ *   q4k_gemm_ggml         q5k_gemm_ggml         q6k_gemm_ggml          (a, b_quant, c, m, n, k)
+ *   q4k_gemm_fused                                                      (a, b_quant, c, m, n, k) */
 TRN_API trn_status trn_module_load_builtin(trn_module* module);
 /* Pointer to and size of that embedded code object (for callers that want trn_module_load_data). */
 TRN_API trn_status trn_builtin_image(const void** image, size_t* size);
@@ -118,6 +119,11 @@ TRN_API trn_status trn_q6k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_d
 TRN_API trn_status trn_q4k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q5k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+
+/* The legacy 18-byte-block "simplified" Q4_K GEMM, kernel name q4k_gemm_fused: W is n rows x (k/32) blocks
+ * (f16 scale + 16 bytes of nibbles, w = scale * q), k a multiple of 32, C as above.  Replaces
+ * QuantizeKernel::new (quantize.rs:84-93, :151-336). */
+TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 
 /* A list of GEMVs issued with one call, in order, on one stream: the weight pass of a decode step
  * (the caller in the reference issues one launch_kernel per matrix per token, docs/roadmaps/
@@ -153,6 +159,8 @@ TRN_API trn_status trn_kquant_gemv_batch(trn_stream stream, const trn_gemv_desc*
 TRN_API trn_status trn_q4k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
 TRN_API trn_status trn_q5k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
 TRN_API trn_status trn_q6k_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy);
+/* out[b*32 + i] = weight i of simplified block b (quantize.rs:237-267). */
+TRN_API trn_status trn_q4k_simplified_dequant_f32(trn_stream stream, trn_dptr out, trn_dptr w, uint64_t n_blocks);
 
 /* ---- 10. timing, errors, tuning (no counterpart in the reference) --------------------------------- */
 TRN_API trn_status trn_event_create(trn_event* event);

@@ -44,6 +44,24 @@ class COracle:
         L.kq_gemv_ref_order_f32.restype = None
         L.kq_gemm_fp64.argtypes = [C.c_int, C.c_int, _u8p, _f32p, C.c_uint32, C.c_uint32, C.c_uint32, _f64p]
         L.kq_gemm_fp64.restype = None
+        L.kq_dequant_simplified.argtypes = [_u8p, C.c_size_t, _f32p]
+        L.kq_dequant_simplified.restype = None
+        L.kq_gemm_simplified_fp64.argtypes = [_u8p, _f32p, C.c_uint32, C.c_uint32, C.c_uint32, _f64p]
+        L.kq_gemm_simplified_fp64.restype = None
+
+    def dequant_simplified(self, buf: np.ndarray) -> np.ndarray:
+        buf = np.ascontiguousarray(buf, np.uint8).reshape(-1)
+        n_blocks = buf.size // 18
+        out = np.empty((n_blocks, 32), np.float32)
+        self.lib.kq_dequant_simplified(_p(buf, _u8p), n_blocks, _p(out, _f32p))
+        return out
+
+    def gemm_simplified_fp64(self, buf, a, m: int, n: int, k: int) -> np.ndarray:
+        buf = np.ascontiguousarray(buf, np.uint8).reshape(-1)
+        a = np.ascontiguousarray(a, np.float32)
+        c = np.empty((m, n), np.float64)
+        self.lib.kq_gemm_simplified_fp64(_p(buf, _u8p), _p(a, _f32p), m, n, k, _p(c, _f64p))
+        return c
 
     def dequant(self, fmt: str, buf: np.ndarray, policy: int = 0) -> np.ndarray:
         buf = np.ascontiguousarray(buf, np.uint8).reshape(-1)

@@ -220,6 +220,33 @@ def dequant_q6k_legacy(buf) -> np.ndarray:
     return (dsc * qf).astype(F32)
 
 
+Q4K_SIMPLE_BLOCK = 32
+Q4K_SIMPLE_BYTES = 18
+
+
+def dequant_q4k_simplified(buf) -> np.ndarray:
+    """Legacy "simplified" Q4_K of q4k_gemm_fused (quantize.rs:41, 151-336): blocks of 32 values in 18
+    bytes - f16 scale at 0 (:237-241), 16 bytes of nibbles at 2 (:250-254); value i sits in byte i/2,
+    low nibble for even i (:245-262); w = scale * q, no min term (:264-267).  Returns [n_blocks, 32] f32."""
+    b = _as_blocks(buf, Q4K_SIMPLE_BYTES)
+    scale = _f16_at(b, 0).astype(np.float32)
+    qs = b[:, 2:18].astype(np.uint32)
+    q = np.empty((b.shape[0], 32), np.uint32)
+    q[:, 0::2] = qs & 15
+    q[:, 1::2] = qs >> 4
+    return (scale[:, None] * q.astype(np.float32)).astype(np.float32)
+
+
+def dequant_matrix_simplified(buf, n: int, k: int) -> np.ndarray:
+    """n rows x (k/32) blocks of 18 bytes, row-major (quantize.rs:225-231) -> f32 [n, k]."""
+    if k % Q4K_SIMPLE_BLOCK:
+        raise ValueError("k must be a multiple of 32")
+    w = dequant_q4k_simplified(buf)
+    if w.shape[0] != n * (k // Q4K_SIMPLE_BLOCK):
+        raise ValueError("buffer size does not match n x k")
+    return w.reshape(n, k)
+
+
 DEQUANT = {
     ("q4k", 0): dequant_q4k, ("q5k", 0): dequant_q5k, ("q6k", 0): dequant_q6k,
     ("q4k", 1): dequant_q4k_legacy, ("q5k", 1): dequant_q5k_legacy, ("q6k", 1): dequant_q6k_legacy,
@@ -311,6 +338,14 @@ def gen_q6k(rng: np.random.Generator, n_sb: int) -> np.ndarray:
     blk[:, 192:208] = rng.integers(-32, 32, (n_sb, 16), dtype=np.int8).view(np.uint8)
     blk[:, 208:210] = _f16_bytes(np.abs(rng.normal(0.0, 0.02, n_sb)))
     return blk.reshape(-1)
+
+
+def gen_q4k_simplified(rng: np.random.Generator, n_blocks: int) -> np.ndarray:
+    """Seeded simplified blocks: scale = f16(|N(0, 0.02)|), nibbles uniform."""
+    b = np.empty((n_blocks, Q4K_SIMPLE_BYTES), np.uint8)
+    b[:, 0:2] = _f16_bytes(np.abs(rng.normal(0.0, 0.02, n_blocks)))
+    b[:, 2:] = rng.integers(0, 256, (n_blocks, 16), dtype=np.uint8)
+    return b.reshape(-1)
 
 
 GEN = {"q4k": gen_q4k, "q5k": gen_q5k, "q6k": gen_q6k}

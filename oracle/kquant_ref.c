@@ -114,6 +114,34 @@ static float dequant_one(int fmt, int policy, const uint8_t* b, unsigned i) {
   return dsc * qf;
 }
 
+/* legacy "simplified" Q4_K block of q4k_gemm_fused: 18 bytes for 32 values, f16 scale at 0 (quantize.rs:237-241),
+ * nibbles at 2, value i in byte i/2, low nibble for even i (:245-262); w = scale * q (:264-267) */
+void kq_dequant_simplified(const uint8_t* w, size_t n_blocks, float* out) {
+  for (size_t b = 0; b < n_blocks; ++b) {
+    const uint8_t* p = w + b * 18u;
+    float scale = f16_to_f32(ld16(p));
+    for (unsigned i = 0; i < 32; ++i) {
+      unsigned q = (p[2u + i / 2u] >> (4u * (i % 2u))) & 0xFu;
+      out[b * 32 + i] = scale * (float)q;
+    }
+  }
+}
+
+/* C[m x n] = A[m x k] . W^T in fp64 on the f32 dequantised simplified weights; c[row*n + col] (:320-327) */
+void kq_gemm_simplified_fp64(const uint8_t* w, const float* a, uint32_t m, uint32_t n, uint32_t k, double* c) {
+  uint32_t nb = k / 32u;
+  for (uint32_t col = 0; col < n; ++col)
+    for (uint32_t r = 0; r < m; ++r) {
+      double acc = 0.0;
+      for (uint32_t b = 0; b < nb; ++b) {
+        float wv[32];
+        kq_dequant_simplified(w + ((size_t)col * nb + b) * 18u, 1, wv);
+        for (unsigned i = 0; i < 32; ++i) acc += (double)wv[i] * (double)a[(size_t)r * k + 32u * b + i];
+      }
+      c[(size_t)r * n + col] = acc;
+    }
+}
+
 void kq_dequant(int fmt, int policy, const uint8_t* w, size_t n_sb, float* out) {
   size_t sb = sb_bytes(fmt);
   for (size_t b = 0; b < n_sb; ++b)

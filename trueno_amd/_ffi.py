@@ -48,10 +48,12 @@ SIGNATURES = {
     "trn_q4k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q5k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q6k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
+    "trn_q4k_gemm_fused": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_kquant_gemv_batch": [vp, vp, C.c_uint32],
     "trn_q4k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q5k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q6k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
+    "trn_q4k_simplified_dequant_f32": [vp, dptr, dptr, C.c_uint64],
     "trn_event_create": [C.POINTER(vp)],
     "trn_event_destroy": [vp],
     "trn_event_record": [vp, vp],

@@ -161,6 +161,51 @@ q4k_gemm_mfma_t2(const uint8_t* planes, const float* meta, const uint8_t* w, flo
 }
 
 // ------------------------------------------------------------------------------------------
+// Legacy "simplified" Q4_K (trueno-gpu/src/kernels/quantize.rs:151-336, kernel name q4k_gemm_fused): blocks of 32
+// values in 18 bytes - f16 scale at 0, 16 bytes of nibbles at 2, value i in byte i/2 (low nibble for even i);
+// w = scale * q, no min term (:237-267).  W is n rows x k/32 blocks, row-major (:225-231); the product is the
+// intended C[m x n] = A[m x k] . W^T, c[row*n + col] (:320-327).  One wave per row of W; lane l takes blocks
+// l, l+64, ...; blockIdx.y walks the rows of A.  Blocks are only 2-byte aligned.
+// ------------------------------------------------------------------------------------------
+extern "C" __global__ void __launch_bounds__(256)
+q4k_gemm_fused(const float* a, const uint8_t* b_quant, float* c, u32 m, u32 n, u32 k) {
+  const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const u32 nb = k >> 5;
+  for (u32 r = blockIdx.y; r < m; r += gridDim.y) {
+    const float* ar = a + static_cast<size_t>(r) * k;
+    for (u32 col = blockIdx.x * waves + wave; col < n; col += gridDim.x * waves) {
+      const uint8_t* rp = b_quant + static_cast<size_t>(col) * nb * 18u;
+      float acc = 0.0f;
+      for (u32 b = lane; b < nb; b += 64u) {
+        const uint8_t* bp = rp + static_cast<size_t>(b) * 18u;
+        const float scale = half_bits_to_f32(static_cast<u32>(bp[0]) | (static_cast<u32>(bp[1]) << 8));
+        float s = 0.0f;
+#pragma unroll
+        for (u32 t = 0; t < 16; ++t) {
+          const u32 byte = bp[2u + t];
+          s = fmaf(static_cast<float>(byte & 15u), ar[32u * b + 2u * t], s);
+          s = fmaf(static_cast<float>(byte >> 4), ar[32u * b + 2u * t + 1u], s);
+        }
+        acc = fmaf(scale, s, acc);
+      }
+      acc = wave_sum(acc);
+      if (lane == 0) c[static_cast<size_t>(r) * n + col] = acc;
+    }
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256)
+q4k_simplified_dequant_f32(float* out, const uint8_t* w, uint64_t n_blocks) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  for (uint64_t gid = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < n_blocks * 32; gid += stride) {
+    const uint8_t* bp = w + (gid >> 5) * 18u;
+    const u32 i = static_cast<u32>(gid & 31u);
+    const float scale = half_bits_to_f32(static_cast<u32>(bp[0]) | (static_cast<u32>(bp[1]) << 8));
+    out[gid] = scale * static_cast<float>((bp[2u + (i >> 1)] >> (4u * (i & 1u))) & 15u);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Dequantise to f32 (test surface): out[sb*256 + i] = w_i.  The fast form shares load/unpack
 // with the GEMV; the generic form takes the decode policy (0 = GEMV family, 1 = GEMM family as
 // written in the reference) and any alignment.

@@ -43,7 +43,7 @@ const char* const kFmtName[NFMT] = {"q4k", "q5k", "q6k"};
 const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 
 // kinds of functions the launch-by-name path recognises
-enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2 };
+enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3 };
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
@@ -64,6 +64,7 @@ struct DeviceKernels {
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
   hipFunction_t gemm_planes = nullptr, gemm_mfma[2] = {};
+  hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
 std::mutex g_mutex;
@@ -125,6 +126,8 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_planes, "kq_gemm_planes")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
+        (e = get_fn(m, &t.dequant_simplified, "q4k_simplified_dequant_f32")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_mfma[0], "q4k_gemm_mfma_t1")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_mfma[1], "q4k_gemm_mfma_t2")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
@@ -260,6 +263,31 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   const uint32_t block = 256, rows_per_block = block / 64;
   const uint32_t grid = std::min<uint32_t>((n + rows_per_block - 1) / rows_per_block, uint32_t(d->cu_count) * 32u);
   return hipModuleLaunchKernel(fn, grid, is_gemv ? 1u : grid_y, 1, block, 1, 1, 0, stream, args, nullptr);
+}
+
+// q4k_gemm_fused: the legacy 18-byte block format (quantize.rs:151-336)
+hipError_t launch_gemm_simplified(hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  if (k % 32u != 0) return hipErrorInvalidValue;
+  if (n == 0 || m == 0) return hipSuccess;
+  if ((a == 0 && k != 0) || c == 0 || (w == 0 && k != 0) || !aligned(a, 4) || !aligned(c, 4)) return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  const uint32_t block = 256, rows_per_block = block / 64;
+  const uint32_t grid = std::min<uint32_t>((n + rows_per_block - 1) / rows_per_block, uint32_t(d->cu_count) * 32u);
+  void* args[] = {&a, &w, &c, &m, &n, &k};
+  return hipModuleLaunchKernel(d->gemm_simplified, grid, std::min<uint32_t>(m, 65535u), 1, block, 1, 1, 0, stream, args, nullptr);
+}
+
+hipError_t launch_dequant_simplified(hipStream_t stream, uint64_t out, uint64_t w, uint64_t n_blocks) {
+  if (n_blocks == 0) return hipSuccess;
+  if (out == 0 || w == 0 || !aligned(out, 4)) return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  const uint32_t grid = uint32_t(std::min<uint64_t>((n_blocks * 32 + 255) / 256, uint64_t(d->cu_count) * 64u));
+  void* args[] = {&out, &w, &n_blocks};
+  return hipModuleLaunchKernel(d->dequant_simplified, grid, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
 }
 
 hipError_t launch_dequant(Fmt f, hipStream_t stream, uint64_t out, uint64_t w, uint64_t n_sb, int policy) {
@@ -628,6 +656,7 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
       if (n == std::string(kFmtName[i]) + "_gemv_warp_reduce") { h->kind = KIND_GEMV; h->fmt = i; }
       if (n == std::string(kFmtName[i]) + "_gemm_ggml") { h->kind = KIND_GEMM; h->fmt = i; }
     }
+    if (n == "q4k_gemm_fused") h->kind = KIND_GEMM_SIMPLIFIED;
   }
   module->functions[name] = h;
   *func = h;
@@ -713,7 +742,7 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
                              void** kernel_params, void** extra) {
   if (!func) return TRN_ERROR_INVALID_VALUE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (func->kind == KIND_GEMV || func->kind == KIND_GEMM) {
+  if (func->kind == KIND_GEMV || func->kind == KIND_GEMM || func->kind == KIND_GEMM_SIMPLIFIED) {
     if (!kernel_params) return TRN_ERROR_INVALID_VALUE;  // the `extra` buffer form is not used by the reference
     for (int i = 0; i < (func->kind == KIND_GEMV ? 5 : 6); ++i)
       if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
@@ -731,6 +760,7 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     std::memcpy(&m, kernel_params[3], 4);
     std::memcpy(&n, kernel_params[4], 4);
     std::memcpy(&k, kernel_params[5], 4);
+    if (func->kind == KIND_GEMM_SIMPLIFIED) return st(launch_gemm_simplified(s, p0, p1, p2, m, n, k));
     return st(launch_gemm_like(Fmt(func->fmt), s, p0, p1, p2, m, n, k, false));
   }
   return st(hipModuleLaunchKernel(func->fn, grid_x, grid_y, grid_z, block_x, block_y, block_z, shared_mem_bytes, s,
@@ -791,6 +821,14 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   return hipModuleLaunchKernel(d->gemv_group, g.first[len], 1, 1, block, 1, 1, lds, stream, args, nullptr);
 }
 }  // namespace
+
+trn_status trn_q4k_gemm_fused(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
+  return st(launch_gemm_simplified(static_cast<hipStream_t>(s), a, b_quant, c, m, n, k));
+}
+
+trn_status trn_q4k_simplified_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w, uint64_t n_blocks) {
+  return st(launch_dequant_simplified(static_cast<hipStream_t>(s), out, w, n_blocks));
+}
 
 trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {
   if (count == 0) return TRN_SUCCESS;

@@ -145,9 +145,9 @@ class _GemmKernel(Kernel):
 
 
 class QuantizeKernel(_GemmKernel):
-    """quantize.rs:66-147.  `QuantizeKernel.ggml(m, n, k)` is the 144-byte super-block format;
-    the plain constructor is the legacy 18-byte "simplified" format, which this backend does not
-    implement (launch raises)."""
+    """quantize.rs:66-147.  `QuantizeKernel.ggml(m, n, k)` is the 144-byte super-block format
+    (q4k_gemm_ggml); the plain constructor is the legacy "simplified" format of 18-byte blocks of 32
+    values (q4k_gemm_fused, quantize.rs:84-93, 151-336)."""
     _SB_BYTES = Q4K_SUPER_BLOCK_BYTES
     _LAUNCHER = "trn_q4k_gemm"
 
@@ -169,15 +169,16 @@ class QuantizeKernel(_GemmKernel):
     def num_blocks_per_row(self) -> int:
         return self.k // self.block_size
 
-    def launch(self, stream, a, b_quant, c) -> None:
-        if self.format is not Q4KFormat.GgmlSuperBlock:
-            raise GpuError("KernelLaunch", "q4k_gemm_fused (18-byte simplified blocks) is not provided by this backend")
-        super().launch(stream, a, b_quant, c)
+    def weight_bytes(self) -> int:
+        if self.format is Q4KFormat.GgmlSuperBlock:
+            return super().weight_bytes()
+        return self.n * self.num_blocks_per_row() * Q4K_BLOCK_BYTES
 
-    def launch_by_name(self, stream, module, a, b_quant, c) -> None:
-        if self.format is not Q4KFormat.GgmlSuperBlock:
-            raise GpuError("FunctionNotFound", "CUDA function 'q4k_gemm_fused' not found in module")
-        super().launch_by_name(stream, module, a, b_quant, c)
+    def launch(self, stream, a, b_quant, c) -> None:
+        if self.format is Q4KFormat.GgmlSuperBlock:
+            return super().launch(stream, a, b_quant, c)
+        _check(_lib().trn_q4k_gemm_fused(stream.raw() if stream is not None else None, _ptr(a), _ptr(b_quant), _ptr(c),
+                                         self.m, self.n, self.k), "KernelLaunch", self.name())
 
 
 class Q5KKernel(_GemmKernel):
@@ -192,6 +193,12 @@ class Q6KKernel(_GemmKernel):
     _NAME = "q6k_gemm_ggml"
     _SB_BYTES = Q6K_SUPER_BLOCK_BYTES
     _LAUNCHER = "trn_q6k_gemm"
+
+
+def dequant_simplified_f32(stream: CudaStream, out, w, n_blocks: int) -> None:
+    """Test surface: out[b*32+i] = weight i of 18-byte simplified block b (quantize.rs:237-267)."""
+    _check(_lib().trn_q4k_simplified_dequant_f32(stream.raw() if stream is not None else None, _ptr(out), _ptr(w), int(n_blocks)),
+           "KernelLaunch", "q4k_simplified_dequant_f32")
 
 
 def dequant_f32(fmt: str, stream: CudaStream, out, w, n_sb: int, policy: int = 0) -> None:
