@@ -8,8 +8,9 @@ pass streams from HBM).  The GEMVs form a dependent chain as in a decoder: q,k,v
 gate,up <- o; down <- gate; next h <- down; head <- h, with h0 ~ N(0,1) and every input
 RMS-normalised.  The list goes to the library in one call (trn_kquant_gemv_batch).  `value` is algorithmic bytes (weights + x + y, each once) over wall time.
 
-Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (the Q4_K GEMV: 192 of the
-225 launches, 2.84 of the 4.13 GB), its launches of one pass timed with HIP events on their stream; `cpu_baseline`: the CPU port
+Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (kq_gemv_group: the fused q,k,v and
+gate,up launches, 64 of the pass's 129 launches, 2.54 of the 4.13 GB), its launches of one pass timed with HIP
+events on their stream; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.
 """
 import argparse
@@ -25,11 +26,11 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per q4k_gemv_flags launch, averaged over the 192 Q4_K launches of the full pass: rocprofv3
+# HBM bytes per kq_gemv_group launch, averaged over the 64 such launches of the full pass: rocprofv3
 # FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the counter reads for kq_copy_u128 on
 # 256 MiB (profiles/kquant_gemv_hbm_traffic_pmc.md).  Counters cannot be read from inside this
 # process, so the figure is carried here and re-measured whenever the kernel changes.
-Q4K_GEMV_TRAFFIC_BYTES_PER_LAUNCH = 14_995_230
+GROUP_TRAFFIC_BYTES_PER_LAUNCH = None
 LAYERS = 32
 SB = {"q4k": 144, "q5k": 176, "q6k": 210}
 LAYER_MATS = [("q", "q4k", 4096, 4096), ("k", "q4k", 4096, 4096), ("v", "q4k", 4096, 4096), ("o", "q4k", 4096, 4096),
@@ -47,6 +48,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the single-launch table of configurations 1, 2, 3 and 5")
     ap.add_argument("--no-executors", action="store_true", help="skip the comparison runs of the opt-in one-launch executors")
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -145,32 +147,39 @@ def main() -> int:
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
     assert np.all(np.isfinite(logits.copy_to_host())), "the pass produced non-finite logits"
 
-    # ---- dominant kernel: the Q4_K GEMV (192 of the 225 launches, 2.84 of the 4.13 GB).  Its launches of one
-    #      pass, in pass order, back to back on the stream, bracketed by HIP events on that stream.
-    q4 = t.GemvBatch()
-    q4_bytes = 0
+    # ---- dominant kernel: kq_gemv_group, the launch that carries the q, k, v projections of a layer (three
+    #      Q4_K 4096x4096 GEMVs on one input) and the one that carries gate and up (two Q4_K 11008x4096): 64 of the
+    #      pass's 129 launches, 2.54 of its 4.13 GB and about 55 % of its GPU time.  Those 64 launches, in pass order,
+    #      back to back on the stream, bracketed by HIP events on that stream.
+    groups = []
+    grp_bytes = 0
     h = h0
     for layer in range(layers):
-        for name, fmt, n, k in LAYER_MATS:
-            if fmt == "q4k":
-                x = h if src_of[name] is None else act[src_of[name]]
-                q4.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
-                q4_bytes += alg_bytes(fmt, n, k)
+        for names in (("q", "k", "v"), ("gate", "up")):
+            g = t.GemvBatch()
+            for name, fmt, n, k in LAYER_MATS:
+                if name in names:
+                    x = h if src_of[name] is None else act[src_of[name]]
+                    g.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
+                    grp_bytes += alg_bytes(fmt, n, k)
+            groups.append(g)
         h = act["down"]
-    n_q4 = len(q4)
+    n_grp = len(groups)
     e0, e1 = ev(), ev()
-    q4_ms = []
+    grp_ms = []
     for _ in range(5):
-        q4.launch(stream)
+        for g in groups:
+            g.launch(stream)
         stream.synchronize()
         L.trn_event_record(e0, stream.raw())
-        q4.launch(stream)
+        for g in groups:
+            g.launch(stream)
         L.trn_event_record(e1, stream.raw())
         stream.synchronize()
-        q4_ms.append(elapsed_ms(e0, e1) / n_q4)
-    q4_ms = sorted(q4_ms)[len(q4_ms) // 2]
-    q4_bytes_per_launch = q4_bytes / n_q4
-    achieved = q4_bytes_per_launch / (q4_ms * 1e-3) / 1e9
+        grp_ms.append(elapsed_ms(e0, e1) / n_grp)
+    grp_ms = sorted(grp_ms)[len(grp_ms) // 2]
+    grp_bytes_per_launch = grp_bytes / n_grp
+    achieved = grp_bytes_per_launch / (grp_ms * 1e-3) / 1e9
 
     # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
     other_modes = {}
@@ -199,8 +208,53 @@ def main() -> int:
         shapes[key] = {"us": round(us, 2), "gbps": round(alg_bytes(fmt, n, k) / us / 1e3, 1),
                        "frac_of_peak": round(alg_bytes(fmt, n, k) / us / 1e3 / HBM_PEAK_GBPS, 4)}
 
+    # ---- the other benchmark configurations, one launch each, cold (16 distinct device copies in rotation) --------
+    configs = {}
+    if not args.no_configs:
+        def timed(launch, reps):
+            for r in range(reps):
+                launch(r)
+            stream.synchronize()
+            L.trn_event_record(e0, stream.raw())
+            for r in range(reps):
+                launch(r)
+            L.trn_event_record(e1, stream.raw())
+            stream.synchronize()
+            return elapsed_ms(e0, e1) * 1e3 / reps
+
+        copies = 16
+        for label, fmt, n, k in (("1_q4k_gemv", "q4k", 4096, 4096), ("2_q6k_gemv", "q6k", 4096, 4096),
+                                 ("2_q6k_gemv", "q6k", 32000, 4096), ("3_q5k_gemv", "q5k", 11008, 4096),
+                                 ("3_q5k_gemv", "q5k", 4096, 11008)):
+            host = kq.gen_matrix(fmt, 1234, n, k)
+            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            xb = xs[0][1 if k == 11008 else 0]
+            fn = getattr(L, f"trn_{fmt}_gemv")
+            us = timed(lambda r: fn(stream.raw(), y[n].as_ptr(), bufs[r % copies].as_ptr(), xb.as_ptr(), k, n), 2 * copies)
+            configs[f"{label}_{n}x{k}"] = {"us": round(us, 2), "gbps": round(alg_bytes(fmt, n, k) / us / 1e3, 1),
+                                            "frac_of_peak": round(alg_bytes(fmt, n, k) / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            for b in bufs:
+                b.free()
+        for n, k in ((14336, 4096), (4096, 14336)):
+            host = kq.gen_matrix("q4k", 1238, n, k)
+            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            for m in (1, 4, 16, 64):
+                a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
+                c = t.GpuBuffer(ctx, m * n, np.float32)
+                us = timed(lambda r: L.trn_q4k_gemm(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k),
+                           2 * copies)
+                nbytes = n * (k // 256) * 144 + 4 * m * k + 4 * m * n
+                configs[f"5_q4k_gemm_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                                       "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                                       "tflops": round(2.0 * m * n * k / us / 1e6, 1)}
+                a.free()
+                c.free()
+            for b in bufs:
+                b.free()
+
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
+    cpu_config1 = None
     if not args.no_cpu_baseline:
         from oracle.cref import CpuBaseline
         cb = CpuBaseline()
@@ -217,6 +271,16 @@ def main() -> int:
             reps += 1
             if time.time() - t_start > 40:
                 break
+        # configuration 1 on the CPU path: dequantise + matvec per call, and matvec on weights dequantised beforehand
+        n1 = k1 = 4096
+        _, sec_dq = cb.dequant_matvec("q4k", host_layer0["q"], hx[k1], k1, n1, cores, 5)
+        w_f32 = kq.dequant_matrix("q4k", host_layer0["q"], n1, k1)
+        _, sec_mv = cb.matvec_f32(w_f32, hx[k1], cores, 5)
+        cpu_config1 = {"shape": "Q4_K 4096x4096", "cores": cores,
+                       "dequant_matvec_us": round(sec_dq / 5 * 1e6, 1),
+                       "dequant_matvec_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_dq / 5) / 1e9, 2),
+                       "matvec_predequantised_f32_us": round(sec_mv / 5 * 1e6, 1),
+                       "matvec_predequantised_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_mv / 5) / 1e9, 2)}
         cpu = {"value": round(layer_bytes * reps / spent / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"layer 0 of the pass (7 GEMVs, {layer_bytes / 1e6:.1f} MB quantized) x {reps} repetitions, "
                          f"dequantise-row + AVX2 dot, {'AVX2+FMA' if cb.has_avx2() else 'scalar'}"}
@@ -232,14 +296,15 @@ def main() -> int:
                                "f32 x and y, RMS-normalised inputs", "gemvs": len(batch), "bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": Q4K_GEMV_TRAFFIC_BYTES_PER_LAUNCH if layers == LAYERS else None,
-                     "kernel": "q4k_gemv_flags", "launches_per_pass": n_q4,
-                     "bytes_per_launch": round(q4_bytes_per_launch), "us_per_launch": round(q4_ms * 1e3, 3)},
+                     "traffic": GROUP_TRAFFIC_BYTES_PER_LAUNCH if layers == LAYERS else None,
+                     "kernel": "kq_gemv_group", "launches_per_pass": n_grp,
+                     "bytes_per_launch": round(grp_bytes_per_launch), "us_per_launch": round(grp_ms * 1e3, 3)},
         "cpu_baseline": cpu,
         "extra": {"us_per_pass": round(ms_per_step * 1e3, 1), "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
                   "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
                   "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes,
+                  "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }
     print(json.dumps(out), flush=True)
