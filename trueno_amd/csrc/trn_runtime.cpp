@@ -60,6 +60,7 @@ struct DeviceKernels {
   hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
   hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr;
   int cooperative = 0;
+  uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
@@ -140,6 +141,9 @@ hipError_t device_kernels(DeviceKernels** out) {
     }
     if (t.cu_count <= 0) t.cu_count = 256;
     (void)hipDeviceGetAttribute(&t.cooperative, hipDeviceAttributeCooperativeLaunch, dev);
+    int occ = 0;
+    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&occ, t.gemv_group, 256, 4096 * 4 + 1024) == hipSuccess && occ >= 1)
+      t.resident_small = uint32_t(std::min(occ, 4));
     t.loaded = true;
     d = t;
   }
@@ -164,7 +168,9 @@ GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint6
   uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : 8u / sw);
   groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
   const uint32_t ug = kGemvRowsPerBatch * groups;
-  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : (sw == 1 ? 4u : 1u);
+  // one-slab kernels: as many workgroups as are resident at once (3 per CU at the kernels' register use; a
+  // fourth per CU would only start when one of the first three has finished)
+  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : (sw == 1 ? d.resident_small : 1u);
   const uint64_t target_blocks = uint64_t(d.cu_count) * per_cu;
   uint64_t rows = (std::max<uint64_t>(n, n_for_rows) + target_blocks - 1) / target_blocks;
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
