@@ -27,8 +27,8 @@
 #include "kquant_quarter.hip.h"
 
 #ifdef CHAIN_TS
-extern __device__ unsigned long long* g_chain_ts;   // [entry][4] for workgroup CHAIN_TS_WG: start, after wait, after x, end
-#define CHAIN_STAMP(slot) do { if (g_chain_ts && blockIdx.x == g_chain_ts_wg && threadIdx.x == 0) g_chain_ts[4 * g_chain_ts_entry + (slot)] = wall_clock64(); } while (0)
+extern __device__ unsigned long long* g_chain_ts;   // [entry][8] for workgroup CHAIN_TS_WG: 0 start, 1 after wait, 2 after x, 3 end, 4 after sum of squares, 5 after row loop
+#define CHAIN_STAMP(slot) do { if (g_chain_ts && blockIdx.x == g_chain_ts_wg && threadIdx.x == 0) g_chain_ts[8 * g_chain_ts_entry + (slot)] = wall_clock64(); } while (0)
 extern __device__ unsigned g_chain_ts_wg;
 static __device__ unsigned g_chain_ts_entry;
 #else
@@ -44,25 +44,22 @@ struct ChainEntry {
 enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u };
 constexpr float kChainNormEps = 1e-6f;
 
-// Sum of squares of the activation vector in ONE fixed order, whatever the launch shape: lane l adds
-// the 16-byte units l, l+64, l+128, ... (x, y, z, w in turn), then the fixed wave butterfly.  Every
-// wave computes it for itself from the staged copy, so no kernel's result depends on its geometry.
+// Sum of squares of the activation vector in ONE fixed order, whatever the launch shape: the vector is cut in
+// groups of 64 16-byte units (256 values); the sum of a group is the fixed wave butterfly over its units (unit
+// 64g + l in lane l, each unit w^2 + (z^2 + (y^2 + x^2)) by FMAs); the groups are added in order.  Any wave can
+// take any group, so the sums are formed while the vector is staged and no kernel's result depends on its
+// geometry.
+__device__ __forceinline__ float unit_sumsq(const f32x4 v) { return fmaf(v.w, v.w, fmaf(v.z, v.z, fmaf(v.y, v.y, v.x * v.x))); }
+
+// the same from a staged copy, by one wave (for engines that stage differently)
 template <class Q>
 __device__ __forceinline__ float canonical_sumsq_lds(const f32x4* lds4, u32 units, u32 lane) {
-  float ss = 0.0f;
-  u32 u = lane;
-  for (; u + 192u < units; u += 256u) {      // four reads in flight; the additions keep their order
-    const f32x4 v0 = lds4[Q::swz(u)], v1 = lds4[Q::swz(u + 64u)], v2 = lds4[Q::swz(u + 128u)], v3 = lds4[Q::swz(u + 192u)];
-    ss = fmaf(v0.x, v0.x, ss); ss = fmaf(v0.y, v0.y, ss); ss = fmaf(v0.z, v0.z, ss); ss = fmaf(v0.w, v0.w, ss);
-    ss = fmaf(v1.x, v1.x, ss); ss = fmaf(v1.y, v1.y, ss); ss = fmaf(v1.z, v1.z, ss); ss = fmaf(v1.w, v1.w, ss);
-    ss = fmaf(v2.x, v2.x, ss); ss = fmaf(v2.y, v2.y, ss); ss = fmaf(v2.z, v2.z, ss); ss = fmaf(v2.w, v2.w, ss);
-    ss = fmaf(v3.x, v3.x, ss); ss = fmaf(v3.y, v3.y, ss); ss = fmaf(v3.z, v3.z, ss); ss = fmaf(v3.w, v3.w, ss);
+  float total = 0.0f;
+  for (u32 g = 0; 64u * g < units; ++g) {
+    const float sg = wave_sum(unit_sumsq(lds4[Q::swz(64u * g + lane)]));
+    total = g == 0u ? sg : total + sg;
   }
-  for (; u < units; u += 64u) {
-    const f32x4 v = lds4[Q::swz(u)];
-    ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
-  }
-  return wave_sum(ss);
+  return total;
 }
 
 // Barrier counters.  Every workgroup adding to one address costs ~15 ns per add at the memory side
@@ -133,7 +130,7 @@ __device__ __forceinline__ u32 chain_prefetch(const ChainEntry& e) {
 }
 
 // One entry on this workgroup's share of rows.  Returns false if the barrier wait gave up.
-//   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][16 floats reduction scratch]
+//   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][k/256 group sums of squares]
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
 template <int FMT, int U, bool COHERENT = false>
 __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
@@ -168,17 +165,13 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
       Q::load(regs[u], col + row * row_bytes, c);
     }
   };
-  if (wave_active) issue(sw, grp);          // in flight across the barrier and the activation staging
-  u32 touched = 0u;
-  if (next) touched = chain_prefetch<U>(*next);
-
-  if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
-  CHAIN_STAMP(1);
-  if (!has_rows) return true;
-
+  // Activations.  Alone on the stream (no barrier to wait for) they are requested BEFORE the weights: loads
+  // return in order, so the vector (an L2 hit) is staged and summed while the weights are still on their way.
+  // Behind a barrier the weights go first, the vector can only be read once the barrier has opened.
   const u32 units = k_dim >> 2;
+  const u32 xgroups = units >> 6;                       // groups of 64 units; k is a multiple of 256
   const f32x4* x4 = reinterpret_cast<const f32x4*>(e.x);
-  for (u32 u = tid; u < units; u += blockDim.x) {
+  auto load_x = [&](u32 u) {
     f32x4 v;
     if constexpr (COHERENT) {
       const u32* xw = reinterpret_cast<const u32*>(e.x) + 4u * u;
@@ -189,14 +182,59 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
     } else {
       v = x4[u];
     }
-    lds4[Q::swz(u)] = v;
+    return v;
+  };
+  constexpr u32 kXPre = 4;                              // groups per wave requested ahead of the weights
+  f32x4 xv[kXPre];
+  const bool x_first = wait_counter == nullptr && has_rows;
+  if (x_first) {
+#pragma unroll
+    for (u32 i = 0; i < kXPre; ++i) {
+      const u32 g = wave + i * waves;
+      xv[i] = load_x(64u * (g < xgroups ? g : 0u) + lane);
+    }
   }
+  // in flight across the barrier and the activation staging.  Issued by every wave, also one without rows
+  // (it reads clamped, valid addresses and ignores them): a branch here would hide the number of loads in
+  // flight from the compiler, which then waits for all of them before the first activation is staged.
+  issue(sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
+  u32 touched = 0u;
+  if (next) touched = chain_prefetch<U>(*next);
+
+  if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
+  CHAIN_STAMP(1);
+  if (!has_rows) return true;
+
   float* part = reinterpret_cast<float*>(lds4 + units);
-  __syncthreads();
+  float* group_ss = part + sw_count * rows_per_block;   // one sum of squares per group of 64 units
+  const bool norm = (e.flags & CHAIN_NORM_INPUT) != 0u;
+  auto stage = [&](u32 g, const f32x4 v) {
+    lds4[Q::swz(64u * g + lane)] = v;
+    if (norm) {
+      const float sg = wave_sum(unit_sumsq(v));
+      if (lane == 0) group_ss[g] = sg;
+    }
+  };
+  if (x_first) {
+#pragma unroll
+    for (u32 i = 0; i < kXPre; ++i) {
+      const u32 g = wave + i * waves;
+      if (g < xgroups) stage(g, xv[i]);
+    }
+  }
+  for (u32 g = wave + (x_first ? kXPre * waves : 0u); g < xgroups; g += waves) stage(g, load_x(64u * g + lane));
+  // Workgroup barrier over the LDS writes only.  __syncthreads() would also drain the weight loads that are in
+  // flight (the compiler waits for every outstanding memory operation before s_barrier), which is the one thing
+  // the ordering above is there to avoid.
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   CHAIN_STAMP(2);
   float scale = 1.0f;
-  if ((e.flags & CHAIN_NORM_INPUT) != 0u)
-    scale = 1.0f / sqrtf(canonical_sumsq_lds<Q>(lds4, units, lane) / static_cast<float>(k_dim) + kChainNormEps);
+  if (norm) {
+    float total = group_ss[0];
+    for (u32 g = 1; g < xgroups; ++g) total += group_ss[g];
+    scale = 1.0f / sqrtf(total / static_cast<float>(k_dim) + kChainNormEps);
+  }
+  CHAIN_STAMP(4);
 
   if (wave_active) {
     for (u32 slab = sw; slab < slabs; slab += sw_count) {
@@ -228,6 +266,7 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
       }
     }
   }
+  CHAIN_STAMP(5);
   __syncthreads();
   for (u32 t = tid; t < rows_per_block; t += blockDim.x) {
     const u32 row = row0 + t;

@@ -34,12 +34,13 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
   const u32 nsb = k_dim >> 8;
   float scale = 1.0f;
   if (flags & CHAIN_NORM_INPUT) {
-    float ss = 0.0f;   // same order as canonical_sumsq_lds: 16-byte units lane, lane+64, ...
-    for (u32 u = lane; u < (k_dim >> 2); u += 64u) {
-      ss = fmaf(x[4 * u], x[4 * u], ss); ss = fmaf(x[4 * u + 1], x[4 * u + 1], ss);
-      ss = fmaf(x[4 * u + 2], x[4 * u + 2], ss); ss = fmaf(x[4 * u + 3], x[4 * u + 3], ss);
+    float total = 0.0f;   // the fixed order of kquant_chain.hip.h: groups of 64 units, butterfly within, in order across
+    for (u32 g = 0; g < nsb; ++g) {
+      const f32x4 v = {x[256u * g + 4u * lane], x[256u * g + 4u * lane + 1u], x[256u * g + 4u * lane + 2u], x[256u * g + 4u * lane + 3u]};
+      const float sg = wave_sum(unit_sumsq(v));
+      total = g == 0u ? sg : total + sg;
     }
-    scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(k_dim) + kChainNormEps);
+    scale = 1.0f / sqrtf(total / static_cast<float>(k_dim) + kChainNormEps);
   }
   for (u32 row = block_id * waves + wave; row < n_dim; row += num_blocks * waves) {
     const uint8_t* rp = w + static_cast<size_t>(row) * nsb * SB;
@@ -71,6 +72,14 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
     chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                          \
+  }                                                                                                      \
+  /* shapes of several slabs (k > 4096) run few waves per CU: four rows in flight per wave instead of two */ \
+  extern "C" __global__ void __launch_bounds__(512)                                                      \
+      fmtname##_gemv_deep(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
+    extern __shared__ f32x4 lds4[];                                                                      \
+    __shared__ u32 s_flag;                                                                               \
+    const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
+    chain_step<FMT, 4>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x); \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \

@@ -352,14 +352,15 @@ __device__ __forceinline__ bool consume_entry(ConsumerState& st, const ChainEntr
     lds_wait();
     if (!consumer_barrier(st.lds_base, st.consumers, st.bar_gen, st.status)) return false;
     if (st.me == 0u) STREAM_STAMP(st.entry_index, 2);
-    // sum of squares in the canonical order (canonical_sumsq_lds of kquant_chain.hip.h), per wave
+    // sum of squares in the fixed order of kquant_chain.hip.h (groups of 64 units), per wave
     float ss = 0.0f;
-    for (u32 u = lane; u < units; u += 64u) {
-      const u32x4 v = lds_ld128(x_lds + 16u * Q::swz(u));
-      const float a = __uint_as_float(v.x), b = __uint_as_float(v.y), c2 = __uint_as_float(v.z), d = __uint_as_float(v.w);
-      ss = fmaf(a, a, ss); ss = fmaf(b, b, ss); ss = fmaf(c2, c2, ss); ss = fmaf(d, d, ss);
+    for (u32 g = 0; 64u * g < units; ++g) {
+      const u32x4 v = lds_ld128(x_lds + 16u * Q::swz(64u * g + lane));
+      const f32x4 f = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+      const float sg = wave_sum(unit_sumsq(f));
+      ss = g == 0u ? sg : ss + sg;
     }
-    st.norm_scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(e.k) + kChainNormEps);
+    st.norm_scale = 1.0f / sqrtf(ss / static_cast<float>(e.k) + kChainNormEps);
   } else {
     // rows shared by several waves reuse the partial-sum slots of the previous entry: everybody must be
     // through with them

@@ -47,8 +47,9 @@ enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED =
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
+constexpr uint32_t kGemvRowsPerBatchDeep = 4; // U of the *_gemv_deep kernels (several slabs)
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
-constexpr uint32_t kLdsScratch = 64;           // reduction scratch at the end of the fast kernels' LDS
+constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
 constexpr uint32_t kFlagNormInput = 1u, kFlagBarrierBefore = 2u, kFlagSameX = 4u;   // CHAIN_* of kquant_chain.hip.h
 // kquant_stream.hip.h: control block, ring (+16 mirror bytes), activations, partial sums, counters
 constexpr uint32_t kStreamCtlBytes = 256, kStreamRingBytes = 96 * 1024, kStreamLdsLimit = 160 * 1024 - 1024;
@@ -57,7 +58,7 @@ struct DeviceKernels {
   bool loaded = false;
   hipModule_t module = nullptr;
   int cu_count = 0;
-  hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
+  hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {}, gemv_deep[NFMT] = {};
   hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
@@ -78,6 +79,7 @@ int g_tune_chain_waves = 0;
 int g_tune_chain_spin_limit = 0;
 int g_tune_chain_prefetch_off = 0;
 int g_tune_stream_consumers = 0;
+int g_tune_deep_off = 0;    // 1: never use the four-rows-in-flight kernels
 int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
 int g_tune_gemm_tiles = 0;      // token tiles (of 8) per wave in the matrix-core GEMM: 1 or 2
@@ -114,6 +116,7 @@ hipError_t device_kernels(DeviceKernels** out) {
       if ((e = get_fn(m, &t.gemv_fast[f], p + "_gemv_warp_reduce")) != hipSuccess ||
           (e = get_fn(m, &t.gemv_flags[f], p + "_gemv_flags")) != hipSuccess ||
           (e = get_fn(m, &t.gemv_generic[f], p + "_gemv_generic")) != hipSuccess ||
+          (e = get_fn(m, &t.gemv_deep[f], p + "_gemv_deep")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_fast[f], p + "_gemm_ggml")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_generic[f], p + "_gemm_generic")) != hipSuccess ||
           (e = get_fn(m, &t.dequant_fast[f], p + "_dequant_f32")) != hipSuccess ||
@@ -156,9 +159,10 @@ hipError_t device_kernels(DeviceKernels** out) {
 struct GemvGeometry {
   uint32_t grid = 0, block = 0, lds = 0;
   bool fits = false;
+  bool deep = false;   // launch the *_gemv_deep kernel
 };
 
-GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint64_t n_for_rows = 0) {
+GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint64_t n_for_rows = 0, bool allow_deep = false) {
   GemvGeometry g;
   const uint32_t nsb = k / 256u;
   const uint32_t slabs = (nsb + 15u) / 16u;
@@ -167,7 +171,8 @@ GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint6
   // slabs every workgroup stages the whole (large) activation vector, so one big workgroup per CU wins.
   uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : 8u / sw);
   groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
-  const uint32_t ug = kGemvRowsPerBatch * groups;
+  g.deep = allow_deep && sw > 1 && !g_tune_deep_off;
+  const uint32_t ug = (g.deep ? kGemvRowsPerBatchDeep : kGemvRowsPerBatch) * groups;
   // one-slab kernels: as many workgroups as are resident at once (3 per CU at the kernels' register use; a
   // fourth per CU would only start when one of the first three has finished)
   const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : (sw == 1 ? d.resident_small : 1u);
@@ -260,9 +265,9 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
   if (k != 0 && gemv_fast_ok(f, c, w, a) && (is_gemv || (aligned(uint64_t(k) * 4u, 16) && aligned(uint64_t(n) * 4u, 4))))
-    g = gemv_geometry(*d, k, n);
+    g = gemv_geometry(*d, k, n, 0, is_gemv);
   if (g.fits) {
-    hipFunction_t fn = is_gemv ? (flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
+    hipFunction_t fn = is_gemv ? (g.deep ? d->gemv_deep[f] : flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
     return hipModuleLaunchKernel(fn, g.grid, is_gemv ? 1u : grid_y, 1, g.block, 1, 1, g.lds, stream, args, nullptr);
   }
   hipFunction_t fn = is_gemv ? d->gemv_generic[f] : d->gemm_generic[f];
@@ -952,6 +957,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "deep_off")) { g_tune_deep_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_tiles_per_wave")) { g_tune_gemm_tiles = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
