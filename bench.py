@@ -4,13 +4,16 @@
 A step is one 7B-style decode weight pass: 32 layers x {Q,K,V,O: Q4_K 4096x4096; gate, up: Q4_K
 11008x4096; down: Q6_K 4096x11008} plus the Q6_K 32000x4096 head - 225 GEMVs over 4.12 GB of
 distinct, seeded synthetic weights resident in HBM (far beyond the 256 MB Infinity Cache, so every
-pass streams from HBM).  The GEMVs form a dependent chain as in a decoder: q,k,v <- h; o <- q;
-gate,up <- o; down <- gate; next h <- down; head <- h, with h0 ~ N(0,1) and every input
-RMS-normalised.  The list goes to the library in one call (trn_kquant_gemv_batch).  `value` is algorithmic bytes (weights + x + y, each once) over wall time.
+pass streams from HBM).  Data flow, per layer: a fresh x_l ~ N(0,1) feeds q, k, v, gate and up; o
+consumes the RMS-normalised output of q; down consumes the RMS-normalised output of gate; the head
+consumes the RMS-normalised output of the last down.  The list goes to the library in one call, in
+layer order (trn_kquant_gemv_batch).  `value` is algorithmic bytes (weights + x + y, each once)
+over wall time.  The same 225 GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h;
+o <- q; gate,up <- o; down <- gate; h <- down) are timed too and reported in `extra`.
 
-Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (kq_gemv_group: the fused q,k,v and
-gate,up launches, 64 of the pass's 129 launches, 2.54 of the 4.13 GB), its launches of one pass timed with HIP
-events on their stream; `cpu_baseline`: the CPU port
+Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (kq_gemv_group: the launches that carry
+up to four independent neighbouring entries, 64 per pass, 3.99 of the 4.13 GB), its launches of one pass timed
+with HIP events on their stream; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.
 """
 import argparse
@@ -85,29 +88,40 @@ def main() -> int:
     ys = {name: t.GpuBuffer(ctx, n, np.float32) for name, _, n, _ in LAYER_MATS}
     print(f"[bench] generated and uploaded {layers} layers in {time.time() - t_gen:.1f} s", file=sys.stderr, flush=True)
 
-    # ---- the pass as one dependent list: per layer  q,k,v <- h ; o <- q ; gate,up <- o ; down <- gate ;
-    #      next h = down ; head <- h.  Every entry normalises its input (RMS, no gain), which keeps the
-    #      chain of random matrices in range.
+    # ---- the pass as one list, in layer order.  Data flow per layer: a fresh x_l ~ N(0,1) feeds q, k, v, gate and
+    #      up; o consumes the RMS-normalised output of q; down consumes the RMS-normalised output of gate; the head
+    #      consumes the RMS-normalised output of the last down.  The library works out from the pointers which
+    #      neighbouring entries are independent of one another.
     NORM = t.GemvBatch.NORM_INPUT
     act = {nm: t.GpuBuffer(ctx, n, np.float32) for nm, n in (("q", 4096), ("k", 4096), ("v", 4096), ("o", 4096),
                                                              ("gate", 11008), ("up", 11008), ("down", 4096))}
-    h0 = xs[0][0]
     logits = y[32000]
-    src_of = {"q": None, "k": None, "v": None, "o": "q", "gate": "o", "up": "o", "down": "gate"}
-    batch = t.GemvBatch()
-    total_bytes = 0
-    weight_bytes = 0
-    h = h0
-    for layer in range(layers):
-        for name, fmt, n, k in LAYER_MATS:
-            x = h if src_of[name] is None else act[src_of[name]]
-            batch.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
-            total_bytes += alg_bytes(fmt, n, k)
-            weight_bytes += n * (k // 256) * SB[fmt]
-        h = act["down"]
-    batch.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, h, NORM)
-    total_bytes += alg_bytes(HEAD[1], HEAD[2], HEAD[3])
-    weight_bytes += HEAD[2] * (HEAD[3] // 256) * SB[HEAD[1]]
+    src_of = {"q": None, "k": None, "v": None, "o": "q", "gate": None, "up": None, "down": "gate"}
+
+    def build_pass(strict):
+        """strict: the serial data flow of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate; h <- down)."""
+        b = t.GemvBatch()
+        nbytes = wbytes = 0
+        h = xs[0][0]
+        for layer in range(layers):
+            for name, fmt, n, k in LAYER_MATS:
+                if strict:
+                    src = {"q": None, "k": None, "v": None, "o": "q", "gate": "o", "up": "o", "down": "gate"}[name]
+                    x, flags = (h if src is None else act[src]), NORM
+                else:
+                    src = src_of[name]
+                    x, flags = (xs[layer][0], 0) if src is None else (act[src], NORM)
+                b.add(fmt, k, n, act[name], weights[layer][name], x, flags)
+                nbytes += alg_bytes(fmt, n, k)
+                wbytes += n * (k // 256) * SB[fmt]
+            h = act["down"]
+        b.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, act["down"], NORM)
+        nbytes += alg_bytes(HEAD[1], HEAD[2], HEAD[3])
+        wbytes += HEAD[2] * (HEAD[3] // 256) * SB[HEAD[1]]
+        return b, nbytes, wbytes
+
+    batch, total_bytes, weight_bytes = build_pass(False)
+    strict_batch, _, _ = build_pass(True)
 
     def ev():
         e = C.c_void_p()
@@ -128,7 +142,7 @@ def main() -> int:
         assert L.trn_event_elapsed_ms(C.byref(ms), a, b) == 0
         return float(ms.value)
 
-    def run_passes(steps, warmup):
+    def run_passes(steps, warmup, batch=batch):
         for _ in range(warmup):
             batch.launch(stream)
         stream.synchronize()
@@ -147,23 +161,30 @@ def main() -> int:
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
     assert np.all(np.isfinite(logits.copy_to_host())), "the pass produced non-finite logits"
 
-    # ---- dominant kernel: kq_gemv_group, the launch that carries the q, k, v projections of a layer (three
-    #      Q4_K 4096x4096 GEMVs on one input) and the one that carries gate and up (two Q4_K 11008x4096): 64 of the
-    #      pass's 129 launches, 2.54 of its 4.13 GB and about 55 % of its GPU time.  Those 64 launches, in pass order,
-    #      back to back on the stream, bracketed by HIP events on that stream.
+    # ---- dominant kernel: kq_gemv_group.  The library fuses neighbouring independent entries (up to four) into one
+    #      launch of this kernel: [q,k,v] of the first layer, then per layer [o,gate,up] and [down, q',k',v' of the
+    #      next layer] - 64 launches that carry all of the pass but the last down and the head (3.99 of 4.13 GB).
+    #      Those 64 launches, in pass order, back to back on the stream, bracketed by HIP events on that stream.
+    entries = []
+    for layer in range(layers):
+        for name, fmt, n, k in LAYER_MATS:
+            src = src_of[name]
+            x, flags = (xs[layer][0], 0) if src is None else (act[src], NORM)
+            entries.append((fmt, k, n, act[name], weights[layer][name], x, flags))
+    cuts = [(0, 3)]
+    for layer in range(layers):
+        base = 7 * layer
+        cuts.append((base + 3, base + 6))
+        if layer + 1 < layers:
+            cuts.append((base + 6, base + 10))
     groups = []
     grp_bytes = 0
-    h = h0
-    for layer in range(layers):
-        for names in (("q", "k", "v"), ("gate", "up")):
-            g = t.GemvBatch()
-            for name, fmt, n, k in LAYER_MATS:
-                if name in names:
-                    x = h if src_of[name] is None else act[src_of[name]]
-                    g.add(fmt, k, n, act[name], weights[layer][name], x, NORM)
-                    grp_bytes += alg_bytes(fmt, n, k)
-            groups.append(g)
-        h = act["down"]
+    for a, b in cuts:
+        g = t.GemvBatch()
+        for fmt, k, n, yb, wb, xb, flags in entries[a:b]:
+            g.add(fmt, k, n, yb, wb, xb, flags)
+            grp_bytes += alg_bytes(fmt, n, k)
+        groups.append(g)
     n_grp = len(groups)
     e0, e1 = ev(), ev()
     grp_ms = []
@@ -180,6 +201,9 @@ def main() -> int:
     grp_ms = sorted(grp_ms)[len(grp_ms) // 2]
     grp_bytes_per_launch = grp_bytes / n_grp
     achieved = grp_bytes_per_launch / (grp_ms * 1e-3) / 1e9
+
+    # ---- the same GEMVs wired as the strictly serial chain of a decoder ------------------------------------
+    strict_ms, _ = run_passes(max(3, args.steps // 2), 2, strict_batch)
 
     # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
     other_modes = {}
@@ -291,9 +315,10 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"7B-style decode weight pass: {layers} layers x (4x Q4_K 4096x4096 + 2x Q4_K 11008x4096 + "
-                               f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} dependent GEMVs "
-                               f"(q,k,v<-h; o<-q; gate,up<-o; down<-gate; h<-down), {total_bytes / 1e9:.3f} GB, batch 1, "
-                               "f32 x and y, RMS-normalised inputs", "gemvs": len(batch), "bytes_per_step": total_bytes},
+                               f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} GEMVs in layer order "
+                               f"(per layer x_l~N(0,1) -> q,k,v,gate,up; o<-norm(q); down<-norm(gate); head<-norm(down)), "
+                               f"{total_bytes / 1e9:.3f} GB, batch 1, f32 x and y", "gemvs": len(batch),
+                               "bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": GROUP_TRAFFIC_BYTES_PER_LAUNCH if layers == LAYERS else None,
@@ -302,6 +327,7 @@ def main() -> int:
         "cpu_baseline": cpu,
         "extra": {"us_per_pass": round(ms_per_step * 1e3, 1), "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
                   "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
+                  "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
                   "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,

@@ -131,8 +131,7 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * format would; a later entry may read what an earlier one wrote (the library finds those
  * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
  * By default the list is issued as one launch per entry, except that up to four neighbouring entries
- * with the same k that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share
- * one launch.  With trn_set_tuning("batch_mode", 1 or 2),
+ * that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share one launch.  With trn_set_tuning("batch_mode", 1 or 2),
  * and when every entry meets the fast kernels' alignment (x 16 B, W 16 B / 2 B for Q6_K), the list
  * runs as ONE cooperative launch of resident workgroups with device-side barriers at the
  * dependencies.  That form keeps, per (device, stream), a small device buffer with the list and its

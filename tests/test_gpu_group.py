@@ -46,7 +46,10 @@ CASES = {
     # mixed formats and ragged row counts in one group; five independent entries (a group holds four)
     "mixed": ([("q4k", 37, 512, "x", "a", 0), ("q5k", 513, 512, "x", "b", 1), ("q6k", 300, 512, "x", "c", 1),
                ("q4k", 64, 512, "x", "d", 0), ("q5k", 129, 512, "x", "e", 1)], 512),
-    # different k next to each other must not be fused; write-after-read must not be fused
+    # different k, formats and row counts in one group (workgroups sized for the widest entry)
+    "mixed_k": ([("q6k", 512, 2816, "x", "a", 1), ("q4k", 1024, 1024, "x", "b", 0), ("q5k", 300, 512, "x", "c", 1),
+                 ("q4k", 37, 4352, "x", "d", 1), ("q6k", 40, 256, "a", "e", 1)], 4352),
+    # write-after-read and read-after-write must not be fused
     "no_fuse": ([("q4k", 512, 512, "x", "a", 1), ("q4k", 256, 768, "x", "b", 1), ("q4k", 512, 512, "a", "x2", 0),
                  ("q4k", 512, 512, "x2", "a", 0)], 768),
 }

@@ -73,14 +73,6 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
     const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
     chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
-  /* shapes of several slabs (k > 4096) run few waves per CU: four rows in flight per wave instead of two */ \
-  extern "C" __global__ void __launch_bounds__(512)                                                      \
-      fmtname##_gemv_deep(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
-    extern __shared__ f32x4 lds4[];                                                                      \
-    __shared__ u32 s_flag;                                                                               \
-    const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
-    chain_step<FMT, 4>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x); \
-  }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
     gemv_generic_body<FMT, POLICY_GEMV>(y, w, x, k_dim, n_dim, blockIdx.x, gridDim.x, flags);            \

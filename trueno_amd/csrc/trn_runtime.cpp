@@ -47,7 +47,6 @@ enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED =
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
-constexpr uint32_t kGemvRowsPerBatchDeep = 4; // U of the *_gemv_deep kernels (several slabs)
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
 constexpr uint32_t kFlagNormInput = 1u, kFlagBarrierBefore = 2u, kFlagSameX = 4u;   // CHAIN_* of kquant_chain.hip.h
@@ -58,7 +57,7 @@ struct DeviceKernels {
   bool loaded = false;
   hipModule_t module = nullptr;
   int cu_count = 0;
-  hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {}, gemv_deep[NFMT] = {};
+  hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
   hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
@@ -79,7 +78,6 @@ int g_tune_chain_waves = 0;
 int g_tune_chain_spin_limit = 0;
 int g_tune_chain_prefetch_off = 0;
 int g_tune_stream_consumers = 0;
-int g_tune_deep_off = 0;    // 1: never use the four-rows-in-flight kernels
 int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
 int g_tune_gemm_tiles = 0;      // token tiles (of 8) per wave in the matrix-core GEMM: 1 or 2
@@ -116,7 +114,6 @@ hipError_t device_kernels(DeviceKernels** out) {
       if ((e = get_fn(m, &t.gemv_fast[f], p + "_gemv_warp_reduce")) != hipSuccess ||
           (e = get_fn(m, &t.gemv_flags[f], p + "_gemv_flags")) != hipSuccess ||
           (e = get_fn(m, &t.gemv_generic[f], p + "_gemv_generic")) != hipSuccess ||
-          (e = get_fn(m, &t.gemv_deep[f], p + "_gemv_deep")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_fast[f], p + "_gemm_ggml")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_generic[f], p + "_gemm_generic")) != hipSuccess ||
           (e = get_fn(m, &t.dequant_fast[f], p + "_dequant_f32")) != hipSuccess ||
@@ -159,10 +156,9 @@ hipError_t device_kernels(DeviceKernels** out) {
 struct GemvGeometry {
   uint32_t grid = 0, block = 0, lds = 0;
   bool fits = false;
-  bool deep = false;   // launch the *_gemv_deep kernel
 };
 
-GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint64_t n_for_rows = 0, bool allow_deep = false) {
+GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n) {
   GemvGeometry g;
   const uint32_t nsb = k / 256u;
   const uint32_t slabs = (nsb + 15u) / 16u;
@@ -171,13 +167,12 @@ GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint6
   // slabs every workgroup stages the whole (large) activation vector, so one big workgroup per CU wins.
   uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : 8u / sw);
   groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
-  g.deep = allow_deep && sw > 1 && !g_tune_deep_off;
-  const uint32_t ug = (g.deep ? kGemvRowsPerBatchDeep : kGemvRowsPerBatch) * groups;
+  const uint32_t ug = kGemvRowsPerBatch * groups;
   // one-slab kernels: as many workgroups as are resident at once (3 per CU at the kernels' register use; a
   // fourth per CU would only start when one of the first three has finished)
   const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : (sw == 1 ? d.resident_small : 1u);
   const uint64_t target_blocks = uint64_t(d.cu_count) * per_cu;
-  uint64_t rows = (std::max<uint64_t>(n, n_for_rows) + target_blocks - 1) / target_blocks;
+  uint64_t rows = (uint64_t(n) + target_blocks - 1) / target_blocks;
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
   // keep activations + partial sums within the LDS the kernel may ask for
   const uint64_t x_bytes = uint64_t(k) * 4u;
@@ -265,9 +260,9 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
   if (k != 0 && gemv_fast_ok(f, c, w, a) && (is_gemv || (aligned(uint64_t(k) * 4u, 16) && aligned(uint64_t(n) * 4u, 4))))
-    g = gemv_geometry(*d, k, n, 0, is_gemv);
+    g = gemv_geometry(*d, k, n);
   if (g.fits) {
-    hipFunction_t fn = is_gemv ? (g.deep ? d->gemv_deep[f] : flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
+    hipFunction_t fn = is_gemv ? (flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
     return hipModuleLaunchKernel(fn, g.grid, is_gemv ? 1u : grid_y, 1, g.block, 1, 1, g.lds, stream, args, nullptr);
   }
   hipFunction_t fn = is_gemv ? d->gemv_generic[f] : d->gemm_generic[f];
@@ -811,25 +806,45 @@ bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) {
          ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
 }
 
-// Entries first .. first+len-1 of a list (len in 2..4, same k, mutually independent, all meeting the fast
-// kernels' preconditions) as ONE launch.
+// Entries first .. first+len-1 of a list (len in 2..4, mutually independent, all meeting the fast kernels'
+// preconditions) as ONE launch.  The workgroups are as large as the largest entry needs (k > 4096 wants one
+// wave per slab of 4096 columns), every entry gets a share of the resident workgroups in proportion to its
+// bytes, and an entry's rows are cut evenly over its share.
 hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gemv_desc* descs, uint32_t len) {
-  uint64_t total_n = 0;
-  for (uint32_t i = 0; i < len; ++i) total_n += descs[i].n;
+  uint32_t waves = 1;
+  double total_bytes = 0.0;
+  for (uint32_t i = 0; i < len; ++i) {
+    const GemvGeometry alone = gemv_geometry(*d, descs[i].k, descs[i].n);
+    if (!alone.fits) return hipErrorInvalidValue;
+    waves = std::max(waves, alone.block / 64u);
+    total_bytes += double(descs[i].n) * (descs[i].k / 256u) * kSbBytes[descs[i].fmt - 4];
+  }
+  // the kernels hold 3 waves per SIMD, 12 per CU
+  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::max(1u, 12u / waves);
+  const double target = double(d->cu_count) * per_cu;
   GemvGroupHost g{};
-  uint32_t block = 0, lds = 0;
+  uint32_t lds = 0;
   g.first[0] = 0;
   for (uint32_t i = 0; i < len; ++i) {
-    const GemvGeometry geo = gemv_geometry(*d, descs[i].k, descs[i].n, total_n);
-    if (!geo.fits) return hipErrorInvalidValue;
-    block = geo.block;
-    lds = std::max(lds, geo.lds);
-    g.e[i] = {descs[i].fmt, descs[i].k, descs[i].n, descs[i].flags, descs[i].w, descs[i].x, descs[i].y};
-    g.first[i + 1] = g.first[i] + geo.grid;
+    const trn_gemv_desc& e = descs[i];
+    const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves), groups = waves / sw;
+    const uint32_t ug = kGemvRowsPerBatch * groups;
+    const double bytes = double(e.n) * nsb * kSbBytes[e.fmt - 4];
+    const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
+    uint64_t rows = (uint64_t(e.n) + share - 1) / share;
+    rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
+    const uint64_t x_bytes = uint64_t(e.k) * 4u;
+    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return hipErrorInvalidValue;
+    const uint64_t max_rows = (kFastLdsLimit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
+    rows = std::min<uint64_t>(rows, max_rows);
+    const uint32_t grid = uint32_t((uint64_t(e.n) + rows - 1) / rows);
+    lds = std::max<uint32_t>(lds, uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch));
+    g.e[i] = {e.fmt, e.k, e.n, e.flags, e.w, e.x, e.y};
+    g.first[i + 1] = g.first[i] + grid;
   }
   g.count = len;
   void* args[] = {&g};
-  return hipModuleLaunchKernel(d->gemv_group, g.first[len], 1, 1, block, 1, 1, lds, stream, args, nullptr);
+  return hipModuleLaunchKernel(d->gemv_group, g.first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
 }
 }  // namespace
 
@@ -858,12 +873,12 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
            gemv_geometry(*dk, d.k, d.n).fits;
   };
   for (uint32_t i = 0; i < count;) {
-    // longest run (up to 4) of entries with the same k that do not touch one another's vectors
+    // longest run (up to 4) of entries that do not touch one another's vectors
     uint32_t len = 1;
     if (!g_tune_group_off && groupable(descs[i])) {
       while (len < 4 && i + len < count) {
         const trn_gemv_desc& c = descs[i + len];
-        bool ok = c.k == descs[i].k && groupable(c);
+        bool ok = groupable(c);
         for (uint32_t j = i; j < i + len && ok; ++j) ok = !gemv_depends(c, descs[j]) && !gemv_depends(descs[j], c);
         if (!ok) break;
         ++len;
@@ -957,7 +972,6 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "deep_off")) { g_tune_deep_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_tiles_per_wave")) { g_tune_gemm_tiles = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
