@@ -14,6 +14,8 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ h16x2 as_h16x2(u32 bits) { return __builtin_bit_cast(h16x2, bits); }
 
 enum : int { FMT_Q4K = 4, FMT_Q5K = 5, FMT_Q6K = 6 };
 enum : int { POLICY_GEMV = 0, POLICY_GEMM_LEGACY = 1 };

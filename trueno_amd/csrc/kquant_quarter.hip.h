@@ -54,25 +54,31 @@ template <> struct Quarter<FMT_Q4K> {
     dm1 = __fmul_rn(dmin, ubyte1(mp));
   }
 
+  // The quants enter the FMAs without an integer-to-float conversion: a 4-bit quant q left in the low bits of a
+  // 16-bit lane IS the f16 subnormal q * 2^-24 (in bits 4..7: q * 2^-20), and v_fma_mix_f32 takes an f16 operand.
+  // One AND therefore prepares two values.  The products and the running sums are the old ones times 2^-24, a
+  // power of two, so every rounding is the same and the factor goes into the scale at the end.
   static __device__ __forceinline__ float dot(const Regs& r, u32 c, const float (&xr)[64], const float (&sx)[NSUM]) {
     float ds0, ds1, dm0, dm1;
     scales(r, c, ds0, ds1, dm0, dm1);
-    float lo = 0.0f, hi = 0.0f;  // hi accumulates 16*q (the high nibble is not shifted down)
+    float lo = 0.0f, hi = 0.0f;  // lo accumulates 2^-24 * q x, hi 2^-20 * q x
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const u32 v = t < 4 ? r.q0[t] : r.q1[t - 4];
-      const u32 l = opaque(v & 0x0F0F0F0Fu), h = opaque(v & 0xF0F0F0F0u);
-      lo = fmaf(ubyte0(l), xr[4 * t + 0], lo);
-      lo = fmaf(ubyte1(l), xr[4 * t + 1], lo);
-      lo = fmaf(ubyte2(l), xr[4 * t + 2], lo);
-      lo = fmaf(ubyte3(l), xr[4 * t + 3], lo);
-      hi = fmaf(ubyte0(h), xr[32 + 4 * t + 0], hi);
-      hi = fmaf(ubyte1(h), xr[32 + 4 * t + 1], hi);
-      hi = fmaf(ubyte2(h), xr[32 + 4 * t + 2], hi);
-      hi = fmaf(ubyte3(h), xr[32 + 4 * t + 3], hi);
+      const u32 w = v >> 8;
+      const h16x2 l02 = as_h16x2(v & 0x000F000Fu), h02 = as_h16x2(v & 0x00F000F0u);   // bytes 0 and 2
+      const h16x2 l13 = as_h16x2(w & 0x000F000Fu), h13 = as_h16x2(w & 0x00F000F0u);   // bytes 1 and 3
+      lo = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], lo);
+      lo = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], lo);
+      lo = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], lo);
+      lo = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], lo);
+      hi = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], hi);
+      hi = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], hi);
+      hi = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], hi);
+      hi = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], hi);
     }
-    float acc = ds0 * lo;
-    acc = fmaf(ds1 * 0.0625f, hi, acc);
+    float acc = (ds0 * 16777216.0f) * lo;
+    acc = fmaf(ds1 * 1048576.0f, hi, acc);
     acc = fmaf(-dm0, sx[0], acc);
     acc = fmaf(-dm1, sx[1], acc);
     return acc;
@@ -229,8 +235,24 @@ template <> struct Quarter<FMT_Q6K> {
     q[3] = opaque(((b >> 4) & 0x0F0F0F0Fu) | ((cc >> 2) & 0x30303030u));
   }
 
-  // (q - 32) is formed before the multiply: summing q*x and correcting by -32*sum(x) afterwards
-  // doubles the rounding error (the two sums are about twice the size of their difference).
+  // Four signed bytes 4*(q - 32) of group g for bytes 4t..4t+3.  q - 32 is the 6-bit two's complement number
+  // q ^ 32; placed in bits 2..7 of a byte its sign-extension is 4*(q - 32), and flipping bit 5 of q is flipping
+  // the high bit of its 2-bit field in qh, which is done once per qh word (`cx` = qh ^ 0xAAAAAAAA).
+  static __device__ __forceinline__ void quants_s4(const Regs& r, int t, u32 cx, u32 (&q)[4]) {
+    const u32 a = r.a[t], b = r.b[t];
+    q[0] = ((a << 2) & 0x3C3C3C3Cu) | ((cx << 6) & 0xC0C0C0C0u);
+    q[1] = ((b << 2) & 0x3C3C3C3Cu) | ((cx << 4) & 0xC0C0C0C0u);
+    q[2] = ((a >> 2) & 0x3C3C3C3Cu) | ((cx << 2) & 0xC0C0C0C0u);
+    q[3] = ((b >> 2) & 0x3C3C3C3Cu) | (cx & 0xC0C0C0C0u);
+  }
+  static __device__ __forceinline__ float sbyte(u32 v, int i) {
+    return static_cast<float>(static_cast<int>(static_cast<int8_t>((v >> (8 * i)) & 0xFFu)));
+  }
+
+  // (q - 32) is formed before the multiply: summing q*x and correcting by -32*sum(x) afterwards doubles the
+  // rounding error (the two sums are about twice the size of their difference).  It enters as the signed byte
+  // 4*(q - 32), converted with its sign in one instruction; the factor 4 is a power of two and leaves through
+  // the scale, so every rounding is what it would be with q - 32 itself.
   static __device__ __forceinline__ float dot(const Regs& r, u32 c, const float (&xr)[64], const float (&sx)[NSUM]) {
     (void)sx;
     float dsc[4];
@@ -239,18 +261,18 @@ template <> struct Quarter<FMT_Q6K> {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       u32 q[4];
-      quants(r, t, q);
+      quants_s4(r, t, r.c[t] ^ 0xAAAAAAAAu, q);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        s[g] = fmaf(ubyte0(q[g]) - 32.0f, xr[16 * g + 4 * t + 0], s[g]);
-        s[g] = fmaf(ubyte1(q[g]) - 32.0f, xr[16 * g + 4 * t + 1], s[g]);
-        s[g] = fmaf(ubyte2(q[g]) - 32.0f, xr[16 * g + 4 * t + 2], s[g]);
-        s[g] = fmaf(ubyte3(q[g]) - 32.0f, xr[16 * g + 4 * t + 3], s[g]);
+        s[g] = fmaf(sbyte(q[g], 0), xr[16 * g + 4 * t + 0], s[g]);
+        s[g] = fmaf(sbyte(q[g], 1), xr[16 * g + 4 * t + 1], s[g]);
+        s[g] = fmaf(sbyte(q[g], 2), xr[16 * g + 4 * t + 2], s[g]);
+        s[g] = fmaf(sbyte(q[g], 3), xr[16 * g + 4 * t + 3], s[g]);
       }
     }
-    float acc = dsc[0] * s[0];
+    float acc = (dsc[0] * 0.25f) * s[0];
 #pragma unroll
-    for (int g = 1; g < 4; ++g) acc = fmaf(dsc[g], s[g], acc);
+    for (int g = 1; g < 4; ++g) acc = fmaf(dsc[g] * 0.25f, s[g], acc);
     return acc;
   }
 
