@@ -59,14 +59,14 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
 }
 
 #define KQ_GEMV_KERNELS(fmtname, FMT)                                                                    \
-  extern "C" __global__ void __launch_bounds__(512)                                                      \
+  extern "C" __global__ void __launch_bounds__(768)                                                      \
       fmtname##_gemv_warp_reduce(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim) {     \
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, 0u, w, x, y};                                               \
     chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, nullptr, nullptr, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
-  extern "C" __global__ void __launch_bounds__(512)                                                      \
+  extern "C" __global__ void __launch_bounds__(768)                                                      \
       fmtname##_gemv_flags(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) {\
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
@@ -90,7 +90,7 @@ struct GemvGroup {
   u32 first[5];      // first[i] .. first[i+1]-1 are the workgroups of entry i
   u32 count;
 };
-extern "C" __global__ void __launch_bounds__(512) kq_gemv_group(const GemvGroup g) {
+extern "C" __global__ void __launch_bounds__(768) kq_gemv_group(const GemvGroup g) {
   extern __shared__ f32x4 lds4[];
   __shared__ u32 s_flag;
   u32 i = 0;

@@ -47,6 +47,7 @@ enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED =
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
+constexpr uint32_t kGemvMaxWaves = 12;        // __launch_bounds__(768) of the fast GEMV kernels
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
 constexpr uint32_t kFlagNormInput = 1u, kFlagBarrierBefore = 2u, kFlagSameX = 4u;   // CHAIN_* of kquant_chain.hip.h
@@ -158,15 +159,16 @@ struct GemvGeometry {
   bool fits = false;
 };
 
-GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n) {
+GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint32_t max_waves = kGemvMaxWaves) {
   GemvGeometry g;
   const uint32_t nsb = k / 256u;
   const uint32_t slabs = (nsb + 15u) / 16u;
-  const uint32_t sw = std::min<uint32_t>(slabs, 8u);
-  // Measured on MI355X: one slab (k <= 4096) runs best as 4 workgroups of 4 waves per CU; with several
-  // slabs every workgroup stages the whole (large) activation vector, so one big workgroup per CU wins.
-  uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : 8u / sw);
-  groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, 8u / sw));
+  const uint32_t sw = std::min<uint32_t>(slabs, max_waves);
+  // Measured on MI355X: one slab (k <= 4096) runs best as workgroups of 4 waves, as many as are resident; with
+  // several slabs every workgroup stages the whole (large) activation vector, so one big workgroup per CU wins
+  // (12 waves: what the kernels' registers let a CU hold).
+  uint32_t groups = g_tune_row_groups > 0 ? uint32_t(g_tune_row_groups) : (sw == 1 ? 4u : max_waves / sw);
+  groups = std::max<uint32_t>(1u, std::min<uint32_t>(groups, max_waves / sw));
   const uint32_t ug = kGemvRowsPerBatch * groups;
   // one-slab kernels: as many workgroups as are resident at once (3 per CU at the kernels' register use; a
   // fourth per CU would only start when one of the first three has finished)
@@ -260,7 +262,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
   if (k != 0 && gemv_fast_ok(f, c, w, a) && (is_gemv || (aligned(uint64_t(k) * 4u, 16) && aligned(uint64_t(n) * 4u, 4))))
-    g = gemv_geometry(*d, k, n);
+    g = gemv_geometry(*d, k, n, is_gemv ? kGemvMaxWaves : 8u);   // the GEMM kernels are built for 8 waves
   if (g.fits) {
     hipFunction_t fn = is_gemv ? (flags ? d->gemv_flags[f] : d->gemv_fast[f]) : d->gemm_fast[f];
     return hipModuleLaunchKernel(fn, g.grid, is_gemv ? 1u : grid_y, 1, g.block, 1, 1, g.lds, stream, args, nullptr);
