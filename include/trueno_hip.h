@@ -131,13 +131,14 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * format would; a later entry may read what an earlier one wrote (the library finds those
  * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
  * By default the list is issued as one launch per entry, except that up to four neighbouring entries
- * that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share one launch.  With trn_set_tuning("batch_mode", 1 or 2),
- * and when every entry meets the fast kernels' alignment (x 16 B, W 16 B / 2 B for Q6_K), the list
- * runs as ONE cooperative launch of resident workgroups with device-side barriers at the
- * dependencies.  That form keeps, per (device, stream), a small device buffer with the list and its
- * barrier counters (allocated on first use, kept until the process ends); a list identical to the
- * previous one on that stream is not uploaded again.  If a device-side wait ever runs out of its
- * (seconds-long) spin budget the kernel exits and the next call on that stream returns
+ * that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share one launch.
+ * With trn_set_tuning("batch_mode", 1 or 2), and when every entry meets the fast kernels' alignment (x 16 B,
+ * W 16 B / 2 B for Q6_K), the list runs as ONE cooperative launch of resident workgroups: the list is cut in
+ * phases of mutually independent entries with a device-side barrier between phases (mode 1), or a producer wave
+ * per CU streams the weights through an LDS ring (mode 2).  These forms keep, per (device, stream), small device
+ * buffers with the list, the work assignment and the barrier counters (allocated on first use, kept until the
+ * process ends); a list identical to the previous one on that stream is not uploaded again.  If a device-side
+ * wait ever runs out of its (seconds-long) spin budget the kernel exits and the next call on that stream returns
  * hipErrorLaunchFailure (719).  All three forms give bit-identical results. */
 #define TRN_GEMV_NORM_INPUT 1u /* the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x */
 typedef struct trn_gemv_desc {
@@ -178,9 +179,11 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * geometry of the single-GEMV kernels.  "batch_mode": how trn_kquant_gemv_batch runs a list - 0 one
  * launch per entry (default), 1 one cooperative launch of resident workgroups with device-side
  * barriers, 2 as 1 with a producer wave per CU streaming the weights through an LDS ring.
- * "chain_blocks_per_cu", "chain_waves", "chain_prefetch_off", "stream_consumers": geometry of modes 1/2.
+ * "stream_consumers": consumer waves of mode 2.
  * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
- * "group_off": 1 = in mode 0 never fuse neighbouring independent entries of a list into one launch. */
+ * "group_off": 1 = in mode 0 never fuse neighbouring independent entries of a list into one launch.
+ * "gemm_mfma_off": 1 = the Q4_K GEMM never takes the matrix-core form; "gemm_tiles_per_wave" (1, 2),
+ * "gemm_k_parts" (1, 2), "gemm_waves" (1..4): its geometry. */
 TRN_API trn_status trn_set_tuning(const char* key, int value);
 
 #ifdef __cplusplus

@@ -66,4 +66,4 @@ def test_stream_equals_per_entry_launches(gpu, case):
         assert np.array_equal(ref[name].view(np.uint32), got[name].view(np.uint32)), (case, name)
     old = _run(gpu, specs2, x_len, {"batch_mode": 1})
     for name in ref:
-        assert np.array_equal(ref[name].view(np.uint32), old[name].view(np.uint32)), (case, name, "resident form")
+        assert np.array_equal(ref[name].view(np.uint32), old[name].view(np.uint32)), (case, name, "resident phases")

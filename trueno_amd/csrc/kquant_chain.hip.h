@@ -1,23 +1,25 @@
-// Persistent executor for an ordered list of k-quant GEMVs (the weight pass of one decode step).
+// The GEMV engine of the fast kernels (chain_step) and the resident executor for an ordered list of k-quant
+// GEMVs (the weight pass of one decode step).
 //
-// Issued one kernel per matrix, a pass is bound by per-launch latency, not by HBM: each launch pays
-// a dispatch gap, an activation-staging phase and a first-load latency during which HBM idles, and a
-// 4096x4096 Q4_K matrix is only ~1.5 us of streaming.  Here the whole list runs in ONE cooperative
-// launch whose workgroups all stay resident:
-//   * every workgroup owns a fixed share of the rows of every entry;
-//   * where an entry reads what an earlier entry wrote, the host marks a device-wide barrier in front
-//     of it; entries between two barriers are independent and stream back to back;
-//   * weights do not depend on activations, so before a workgroup waits at a barrier it has already
-//     requested the first rows of the next entry - HBM keeps streaming across the dependency;
-//   * the barrier is a (two-level) counter in device memory: atomic add to arrive, bounded spin to
-//     leave.  A spin that runs out sets a status word and every workgroup exits; nothing can hang.
-//   * the only data that crosses workgroups are the activation vectors and the counters.  The L2s of
-//     the eight XCDs are not coherent with each other for ordinary accesses, and the release/acquire
-//     fences that would make them so write back / invalidate whole caches (tens of microseconds per
-//     barrier, measured).  Instead exactly those accesses are made coherent: y is stored and x is
-//     loaded with agent-scope atomic (relaxed) accesses, which go to the memory side; weights are
-//     read-only and keep the fast path.
-// The per-row arithmetic is the quarter-block engine of kquant_quarter.hip.h, unchanged.
+// chain_step computes one workgroup's share of the rows of one matrix: it stages the activation vector in LDS,
+// keeps each lane's 64 activations in registers and streams the rows (kquant_quarter.hip.h has the per-row
+// arithmetic).  The single-GEMV kernels, the grouped launch and the resident executor all call it, so they give
+// the same bits.
+//
+// Resident executor (phases_body, at the end of this file): the whole list in ONE cooperative launch whose
+// workgroups all stay resident.
+//   * the host cuts the list into phases of mutually independent entries and deals the workgroups of a phase to
+//     its entries in proportion to their bytes;
+//   * between phases there is a device-wide barrier: a (two-level) counter in device memory, atomic add to
+//     arrive, bounded spin to leave.  A spin that runs out sets a status word and every workgroup exits;
+//     nothing can hang;
+//   * weights do not depend on activations, so before a workgroup waits at a barrier it has already requested
+//     the first rows of its next entry;
+//   * the only data that crosses workgroups are the activation vectors and the counters.  The L2s of the eight
+//     XCDs are not coherent with each other for ordinary accesses, and the release/acquire fences that would
+//     make them so write back / invalidate whole caches (tens of microseconds per barrier, measured).  Instead
+//     exactly those accesses are made coherent: y is stored and x is loaded with agent-scope atomic (relaxed)
+//     accesses, which go to the memory side; weights are read-only and keep the fast path.
 //
 // CHAIN_NORM_INPUT: the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x (an RMS normalisation
 // without gain, applied as one factor on y; every workgroup stages all of x anyway).  It keeps a
@@ -102,40 +104,12 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
   return *s_flag != 0u;
 }
 
-// Touches one dword in every 128-byte line of this workgroup's share of rows of entry `e` (capped),
-// so the lines are on their way into this XCD's L2 while the workgroup waits at a barrier or works
-// on the current entry.  The loaded words are returned so the loads stay live; the caller folds
-// them into a value it never stores.
-constexpr u32 kChainPrefetchLoads = 3u;         // per thread
-constexpr u32 kChainPrefetchLine = 128u;
-template <int U>
-__device__ __forceinline__ u32 chain_prefetch(const ChainEntry& e) {
-  const u32 nsb = e.k >> 8;
-  const u32 sbb = e.fmt == FMT_Q4K ? 144u : e.fmt == FMT_Q5K ? 176u : 210u;
-  u32 rows_per_block = (e.n + gridDim.x - 1) / gridDim.x;
-  rows_per_block = ((rows_per_block + U - 1) / U) * U;
-  const u32 row0 = blockIdx.x * rows_per_block;
-  if (row0 >= e.n || nsb == 0) return 0u;
-  const u32 rows = min(rows_per_block, e.n - row0);
-  const size_t row_bytes = static_cast<size_t>(nsb) * sbb;
-  const size_t bytes = static_cast<size_t>(rows) * row_bytes;
-  const uint8_t* base = e.w + static_cast<size_t>(row0) * row_bytes;
-  u32 acc = 0u;
-#pragma unroll
-  for (u32 i = 0; i < kChainPrefetchLoads; ++i) {
-    const size_t off = (static_cast<size_t>(i) * blockDim.x + threadIdx.x) * kChainPrefetchLine;
-    if (off + 4 <= bytes) acc ^= *reinterpret_cast<const u32*>(base + (off & ~static_cast<size_t>(3)));
-  }
-  return acc;
-}
-
 // One entry on this workgroup's share of rows.  Returns false if the barrier wait gave up.
 //   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][k/256 group sums of squares]
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
 template <int FMT, int U, bool COHERENT = false>
 __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
-                                           f32x4* lds4, u32* s_flag, const ChainEntry* next, u32* sink,
-                                           u32 block_id, u32 num_blocks) {
+                                           f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks) {
   using Q = Quarter<FMT>;
   const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
@@ -198,8 +172,6 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   // (it reads clamped, valid addresses and ignores them): a branch here would hide the number of loads in
   // flight from the compiler, which then waits for all of them before the first activation is staged.
   issue(sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
-  u32 touched = 0u;
-  if (next) touched = chain_prefetch<U>(*next);
 
   if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
   CHAIN_STAMP(1);
@@ -280,32 +252,57 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
         e.y[row] = s * scale;
     }
   }
-  if (sink && touched == 0x9E3779B9u) *sink = touched;   // keeps the prefetch loads; practically never taken
   CHAIN_STAMP(3);
   return true;
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Phase executor: the whole list in one resident launch of ONE workgroup per CU.  The host cuts the list into
+// phases of mutually independent entries and, per phase, deals the workgroups to the entries in proportion to
+// their bytes (PhaseAssign, one per phase and workgroup).  A workgroup computes its share of its entry exactly
+// as a separate launch would, with a device-wide barrier between phases.  The loop over phases is written per
+// format (a workgroup stays in one format's loop for as long as its assignments keep that format): with the
+// three engines side by side in one loop body the register allocator needs half again as many registers.
+// ------------------------------------------------------------------------------------------------------------
+struct PhaseAssign {
+  u32 entry;        // index into the entry list
+  u32 block_id;     // this workgroup's index among the num_blocks workgroups of that entry
+  u32 num_blocks;
+  u32 fmt;          // format of that entry; 0 = this workgroup has nothing to do in this phase
+};
+
+template <int FMT, int U>
+__device__ __forceinline__ u32 phases_run(u32 p, const ChainEntry* __restrict__ entries, const PhaseAssign* __restrict__ assign,
+                                          u32 phases, u32* counters, u32* status, u32 spin_limit, f32x4* lds4, u32* s_flag) {
+  const u32 stride = chain_barrier_stride(gridDim.x);
+  for (; p < phases; ++p) {
+    const PhaseAssign a = assign[static_cast<size_t>(p) * gridDim.x + blockIdx.x];
+    if (a.fmt != static_cast<u32>(FMT)) break;
+    const ChainEntry e = entries[a.entry];
+    if (!chain_step<FMT, U, true>(e, p ? counters + p * stride : nullptr, spin_limit, status, lds4, s_flag, a.block_id, a.num_blocks))
+      return 0xFFFFFFFFu;
+    if (p + 1 < phases) chain_arrive(counters + (p + 1) * stride);
+    else __syncthreads();
+  }
+  return p;
+}
+
 template <int U>
-__device__ __forceinline__ void chain_body(const ChainEntry* __restrict__ entries, u32 count, u32* counters,
-                                           u32* status, u32 spin_limit, u32 prefetch) {
+__device__ __forceinline__ void phases_body(const ChainEntry* __restrict__ entries, const PhaseAssign* __restrict__ assign,
+                                            u32 phases, u32* counters, u32* status, u32 spin_limit) {
   extern __shared__ f32x4 lds4[];
   __shared__ u32 s_flag;
-  u32 bar = 0;
-  for (u32 i = 0; i < count; ++i) {
-#ifdef CHAIN_TS
-    if (threadIdx.x == 0 && blockIdx.x == g_chain_ts_wg) g_chain_ts_entry = i;
-#endif
-    const ChainEntry e = entries[i];
-    u32* wait_counter = (e.flags & CHAIN_BARRIER_BEFORE) ? counters + bar * chain_barrier_stride(gridDim.x) : nullptr;
-    bool ok = true;
-    const ChainEntry* next = (prefetch && i + 1 < count) ? entries + i + 1 : nullptr;
-    if (e.fmt == FMT_Q4K) ok = chain_step<FMT_Q4K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
-    else if (e.fmt == FMT_Q5K) ok = chain_step<FMT_Q5K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
-    else if (e.fmt == FMT_Q6K) ok = chain_step<FMT_Q6K, U, true>(e, wait_counter, spin_limit, status, lds4, &s_flag, next, status + 1, blockIdx.x, gridDim.x);
-    if (!ok) return;
-    if (wait_counter) ++bar;
-    const bool arrive = i + 1 < count && (entries[i + 1].flags & CHAIN_BARRIER_BEFORE) != 0u;
-    if (arrive) chain_arrive(counters + bar * chain_barrier_stride(gridDim.x));
-    else __syncthreads();                  // LDS is reused by the next entry
+  const u32 stride = chain_barrier_stride(gridDim.x);
+  u32 p = 0;
+  while (p < phases) {
+    const u32 fmt = assign[static_cast<size_t>(p) * gridDim.x + blockIdx.x].fmt;
+    if (fmt == FMT_Q4K) p = phases_run<FMT_Q4K, U>(p, entries, assign, phases, counters, status, spin_limit, lds4, &s_flag);
+    else if (fmt == FMT_Q5K) p = phases_run<FMT_Q5K, U>(p, entries, assign, phases, counters, status, spin_limit, lds4, &s_flag);
+    else if (fmt == FMT_Q6K) p = phases_run<FMT_Q6K, U>(p, entries, assign, phases, counters, status, spin_limit, lds4, &s_flag);
+    else {                                   // idle in this phase: keep the barriers in step
+      if (p && !chain_wait(counters + p * stride, spin_limit, status, &s_flag)) return;
+      if (p + 1 < phases) chain_arrive(counters + (p + 1) * stride);
+      ++p;
+    }
   }
 }

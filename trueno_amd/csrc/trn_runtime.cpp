@@ -59,7 +59,7 @@ struct DeviceKernels {
   hipModule_t module = nullptr;
   int cu_count = 0;
   hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
-  hipFunction_t chain = nullptr, stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr;
+  hipFunction_t stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr, phases = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
@@ -73,11 +73,8 @@ std::mutex g_mutex;
 DeviceKernels g_dev[kMaxDevices];
 int g_tune_blocks_per_cu = 0;
 int g_tune_row_groups = 0;
-int g_tune_batch_mode = 0;   // 0: one launch per entry (default); 1: resident workgroups + barriers; 2: 1 + streaming producer
-int g_tune_chain_blocks_per_cu = 0;
-int g_tune_chain_waves = 0;
+int g_tune_batch_mode = 0;   // 0: launches (default); 1: resident phases + barriers; 2: resident, streaming producer wave
 int g_tune_chain_spin_limit = 0;
-int g_tune_chain_prefetch_off = 0;
 int g_tune_stream_consumers = 0;
 int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
@@ -124,9 +121,9 @@ hipError_t device_kernels(DeviceKernels** out) {
       }
     }
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
-        (e = get_fn(m, &t.chain, "kq_gemv_chain")) != hipSuccess ||
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
+        (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_planes, "kq_gemm_planes")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
         (e = get_fn(m, &t.dequant_simplified, "q4k_simplified_dequant_f32")) != hipSuccess ||
@@ -332,6 +329,10 @@ struct ChainWorkspace {
   uint32_t* d_status = nullptr;
   std::vector<ChainEntryHost> last;
   uint32_t grid = 0, block = 0, lds = 0, barriers = 0;
+  // phase executor: per phase and workgroup, what to do (PhaseAssign of kquant_chain.hip.h)
+  void* d_assign = nullptr;
+  size_t cap_assign = 0;
+  std::vector<uint32_t> last_assign;
 };
 std::map<std::pair<int, hipStream_t>, ChainWorkspace> g_chain_ws;
 
@@ -340,6 +341,127 @@ std::map<std::pair<int, hipStream_t>, ChainWorkspace> g_chain_ws;
 uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u + (num_workgroups + 31u) / 32u); }
 
 bool ranges_overlap(uint64_t a, uint64_t alen, uint64_t b, uint64_t blen) { return a < b + blen && b < a + alen; }
+
+bool desc_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) {
+  return ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
+         ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
+}
+
+// batch_mode 1: the list as phases of independent entries in ONE resident launch (kq_gemv_phases): one workgroup
+// of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
+// barrier between phases.  *handled = false (and hipSuccess): not possible here, issue the list the plain way.
+hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t stream, const trn_gemv_desc* descs,
+                         uint32_t count, bool* handled) {
+  constexpr uint32_t kWaves = kGemvMaxWaves, kMaxPerPhase = 16;
+  const uint32_t G = uint32_t(d->cu_count);
+  // phases: a new one starts where an entry touches a vector of an entry of the current phase
+  std::vector<std::pair<uint32_t, uint32_t>> ph;
+  uint32_t begin = 0;
+  for (uint32_t i = 0; i < count; ++i) {
+    bool dep = i - begin >= kMaxPerPhase || i - begin >= G;
+    for (uint32_t j = begin; j < i && !dep; ++j) dep = desc_depends(descs[i], descs[j]) || desc_depends(descs[j], descs[i]);
+    if (dep) {
+      ph.emplace_back(begin, i);
+      begin = i;
+    }
+  }
+  ph.emplace_back(begin, count);
+  const uint32_t phases = uint32_t(ph.size());
+  std::vector<uint32_t> assign(size_t(phases) * G * 4u, 0u);   // entry, block_id, num_blocks, fmt
+  std::vector<ChainEntryHost> entries(count);
+  for (uint32_t i = 0; i < count; ++i) entries[i] = {descs[i].fmt, descs[i].k, descs[i].n, descs[i].flags, descs[i].w, descs[i].x, descs[i].y};
+  uint32_t lds = 0;
+  for (uint32_t p = 0; p < phases; ++p) {
+    const uint32_t a = ph[p].first, b = ph[p].second, m = b - a;
+    double total = 0.0;
+    std::vector<double> bytes(m);
+    for (uint32_t i = 0; i < m; ++i) {
+      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4];
+      total += bytes[i];
+    }
+    // shares: at least one workgroup each, the rest in proportion to the bytes (largest remainders first)
+    std::vector<uint32_t> share(m, 1u);
+    uint32_t left = G - m;
+    std::vector<std::pair<double, uint32_t>> frac(m);
+    for (uint32_t i = 0; i < m; ++i) {
+      const double want = double(G - m) * bytes[i] / total;
+      const uint32_t whole = uint32_t(want);
+      share[i] += whole;
+      left -= whole;
+      frac[i] = {want - whole, i};
+    }
+    std::sort(frac.begin(), frac.end(), [](const auto& x, const auto& y) { return x.first > y.first; });
+    for (uint32_t i = 0; i < left; ++i) ++share[frac[i % m].second];
+    uint32_t wg = 0;
+    for (uint32_t i = 0; i < m; ++i) {
+      const trn_gemv_desc& e = descs[a + i];
+      const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, kWaves), groups = kWaves / sw;
+      const uint32_t ug = kGemvRowsPerBatch * groups;
+      uint64_t rows = (uint64_t(e.n) + share[i] - 1) / share[i];
+      rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
+      const uint64_t need = uint64_t(e.k) * 4u + uint64_t(sw) * rows * 4u + kLdsScratch;
+      if (need > kFastLdsLimit) return hipSuccess;
+      lds = std::max<uint32_t>(lds, uint32_t(need));
+      const uint32_t used = uint32_t((uint64_t(e.n) + rows - 1) / rows);
+      for (uint32_t bId = 0; bId < share[i]; ++bId, ++wg) {
+        uint32_t* q = &assign[(size_t(p) * G + wg) * 4u];
+        if (bId < used) { q[0] = a + i; q[1] = bId; q[2] = used; q[3] = e.fmt; }
+      }
+    }
+  }
+  int occ = 0;
+  if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&occ, d->phases, int(64u * kWaves), lds) != hipSuccess || occ < 1)
+    return hipSuccess;
+  hipError_t err;
+  const bool same = ws->last.size() == entries.size() && ws->last_assign == assign &&
+                    std::memcmp(ws->last.data(), entries.data(), entries.size() * sizeof(ChainEntryHost)) == 0;
+  if (!same) {
+    if ((err = hipStreamSynchronize(stream)) != hipSuccess) return err;  // a list in flight may still read the device copies
+    if (ws->cap_entries < entries.size()) {
+      if (ws->d_entries) (void)hipFree(ws->d_entries);
+      ws->d_entries = nullptr;
+      ws->cap_entries = 0;
+      if ((err = hipMalloc(&ws->d_entries, entries.size() * sizeof(ChainEntryHost))) != hipSuccess) return err;
+      ws->cap_entries = entries.size();
+    }
+    if (ws->cap_assign < assign.size()) {
+      if (ws->d_assign) (void)hipFree(ws->d_assign);
+      ws->d_assign = nullptr;
+      ws->cap_assign = 0;
+      if ((err = hipMalloc(&ws->d_assign, assign.size() * sizeof(uint32_t))) != hipSuccess) return err;
+      ws->cap_assign = assign.size();
+    }
+    if ((err = hipMemcpy(ws->d_entries, entries.data(), entries.size() * sizeof(ChainEntryHost), hipMemcpyHostToDevice)) != hipSuccess ||
+        (err = hipMemcpy(ws->d_assign, assign.data(), assign.size() * sizeof(uint32_t), hipMemcpyHostToDevice)) != hipSuccess)
+      return err;
+    ws->last = entries;
+    ws->last_assign = assign;
+  }
+  const size_t n_words = size_t(phases + 1u) * chain_barrier_stride_host(G);
+  if (ws->cap_counters < n_words) {
+    if ((err = hipStreamSynchronize(stream)) != hipSuccess) return err;
+    if (ws->d_counters) (void)hipFree(ws->d_counters);
+    ws->d_counters = nullptr;
+    ws->cap_counters = 0;
+    if ((err = hipMalloc(reinterpret_cast<void**>(&ws->d_counters), n_words * sizeof(uint32_t))) != hipSuccess) return err;
+    ws->cap_counters = n_words;
+  }
+  uint32_t n_counters = uint32_t(n_words), zero = 0u;
+  void* fill_args[] = {&ws->d_counters, &n_counters, &zero};
+  const uint32_t fill_grid = std::max(1u, std::min(64u, (n_counters + 255u) / 256u));
+  if ((err = hipModuleLaunchKernel(d->fill_u32, fill_grid, 1, 1, 256, 1, 1, 0, stream, fill_args, nullptr)) != hipSuccess) return err;
+  uint32_t spin_limit = g_tune_chain_spin_limit > 0 ? uint32_t(g_tune_chain_spin_limit) : 4000000u;
+  uint32_t np = phases;
+  void* args[] = {&ws->d_entries, &ws->d_assign, &np, &ws->d_counters, &ws->d_status, &spin_limit};
+  err = hipModuleLaunchCooperativeKernel(d->phases, G, 1, 1, 64u * kWaves, 1, 1, lds, stream, args);
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    return hipSuccess;
+  }
+  ws->grid = G; ws->block = 64u * kWaves; ws->lds = lds; ws->barriers = phases;
+  *handled = true;
+  return hipSuccess;
+}
 
 // Runs the list as one cooperative launch when every entry qualifies for the fast kernels.
 // *handled = false (and hipSuccess) means the caller should issue the entries one by one.
@@ -390,6 +512,8 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
     ws->h_status[0] = 0;
     return hipErrorLaunchFailure;
   }
+
+  if (g_tune_batch_mode != 2) return launch_phases(d, ws, stream, descs, count, handled);
 
   // ---- streaming form: one workgroup per CU, a producer wave feeding an LDS ring -------------------
   bool use_stream = g_tune_batch_mode == 2;
@@ -462,61 +586,9 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
       return hipSuccess;
     }
     (void)hipGetLastError();   // not launchable in this form here: try the plain resident form below
-    for (auto& en : entries) en.flags &= ~kFlagSameX;
-  } else {
-    for (auto& en : entries) en.flags &= ~kFlagSameX;
   }
 
-  // wave count per workgroup: the one that leaves the fewest waves idle, weighted by bytes
-  uint32_t waves = uint32_t(g_tune_chain_waves);
-  if (waves == 0) {
-    double best = -1.0;
-    for (uint32_t cand : {6u, 8u, 4u}) {
-      double useful = 0.0, total = 0.0;
-      for (uint32_t i = 0; i < count; ++i) {
-        const uint32_t slabs = (descs[i].k / 256u + 15u) / 16u, sw = std::min(slabs, cand);
-        const double bytes = double(descs[i].n) * descs[i].k;
-        useful += bytes * double(sw * (cand / sw)) / cand;
-        total += bytes;
-      }
-      if (useful / total > best + 1e-9) { best = useful / total; waves = cand; }
-    }
-  }
-  waves = std::max(1u, std::min(waves, 8u));
-  const uint32_t block = 64u * waves;
-  auto lds_for = [&](uint32_t grid) {
-    uint32_t lds = 0;
-    for (uint32_t i = 0; i < count; ++i) {
-      const uint32_t slabs = (descs[i].k / 256u + 15u) / 16u, sw = std::min(slabs, waves);
-      uint64_t rows = (uint64_t(descs[i].n) + grid - 1) / grid;
-      rows = (rows + kGemvRowsPerBatch - 1) / kGemvRowsPerBatch * kGemvRowsPerBatch;
-      const uint64_t need = uint64_t(descs[i].k) * 4u + uint64_t(sw) * rows * 4u + kLdsScratch;
-      if (need > kFastLdsLimit) return 0u;
-      lds = std::max<uint32_t>(lds, uint32_t(need));
-    }
-    return lds;
-  };
-  uint32_t lds = lds_for(uint32_t(d->cu_count));
-  if (lds == 0) return hipSuccess;
-  int per_cu = 0;
-  if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, d->chain, int(block), lds) != hipSuccess || per_cu < 1)
-    return hipSuccess;
-  if (g_tune_chain_blocks_per_cu > 0) per_cu = std::min(per_cu, g_tune_chain_blocks_per_cu);
-  per_cu = std::min(per_cu, 2);  // barrier cost grows with the number of workgroups
-  const uint32_t grid = uint32_t(d->cu_count) * uint32_t(per_cu);
-  lds = lds_for(grid);
-
-  if ((e = upload(grid)) != hipSuccess) return e;
-  ws->grid = grid; ws->block = block; ws->lds = lds; ws->barriers = barriers;
-  uint32_t prefetch = g_tune_chain_prefetch_off ? 0u : 1u;
-  void* args[] = {&ws->d_entries, &cnt, &ws->d_counters, &ws->d_status, &spin_limit, &prefetch};
-  e = hipModuleLaunchCooperativeKernel(d->chain, grid, 1, 1, block, 1, 1, lds, stream, args);
-  if (e != hipSuccess) {
-    (void)hipGetLastError();
-    return hipSuccess;  // not launchable as one resident grid here: the caller issues the entries one by one
-  }
-  *handled = true;
-  return hipSuccess;
+  return launch_phases(d, ws, stream, descs, count, handled);
 }
 
 }  // namespace
@@ -968,10 +1040,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemv_blocks_per_cu")) { g_tune_blocks_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_row_groups")) { g_tune_row_groups = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "batch_mode")) { g_tune_batch_mode = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "chain_blocks_per_cu")) { g_tune_chain_blocks_per_cu = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "chain_waves")) { g_tune_chain_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "chain_spin_limit")) { g_tune_chain_spin_limit = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "chain_prefetch_off")) { g_tune_chain_prefetch_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
