@@ -1,0 +1,406 @@
+// Batched Q4_K GEMM on the matrix cores (gfx950, v_mfma_f32_32x32x16_f16).
+//
+//   C[m x n] = A[m x k] . dequant(W[n x k])^T,  c[row*n + col]      (trueno-gpu/src/kernels/quantize.rs:568-574,
+//   decode of the weights as in the GEMV family, quantize.rs:1237-1483)
+//
+// f16 operands without giving up f32 accuracy:
+//   * the weight operand is  q * s_j * 2^-14  (nibble q <= 15, 6-bit sub-block scale s_j <= 63): an integer
+//     below 1024 times a power of two, exact in f16.  It costs one AND and one packed multiply per two weights:
+//     a nibble left in place in a 16-bit lane is the f16 subnormal q * 2^-24 (bits 4..7: q * 2^-20), and the
+//     packed multiply by s_j * 2^10 (s_j * 2^6) turns it into the normal number wanted;
+//   * every (token, super-block) run of 256 activations is scaled by a power of two so that its largest
+//     element lies in [2^14, 2^15) and each element is split in two f16 pieces, hi = f16(a),
+//     lo = f16((a - hi) * 2^11): 22 bits and a sign per element, products exact in the matrix cores' f32
+//     accumulators.  The pieces are two rows of the token operand, so a tile of 32 operand rows is 16 tokens.
+//     The workgroup does this itself, one super-block ahead of the products, straight into LDS;
+//   * the accumulators run over a whole super-block (the sub-block scales are inside the operand), then
+//     tot += d * 2^E(token, super-block) * acc per (row, token, super-block);
+//   * the min term  dmin * sum_j m_j * (sum of a over sub-block j)  is one more small product per super-block
+//     (v_mfma_f32_32x32x8_f16: m_j against the sub-block sums, split in two pieces like a).
+//
+// Operand roles: A operand = token pieces (row 2*token + piece), B operand = 32 rows of W.  Lane l supplies
+// A[row l%32][8 k-slots of group l/32] and B[the same k-slots][col l%32]; D[row 8*(v/4) + 4*(l/32) + v%4][col l%32]
+// arrives in lane l, register v.  Which k a slot stands for is this file's choice (both operands use the same
+// table): lane group g = l/32 of W row r takes the 64 bytes qs[64g .. 64g+63] of a super-block, i.e. its
+// sub-blocks 4g .. 4g+3; product q = 2u + h (u = 0..7, h = 0 low / 1 high nibbles) takes bytes 8u .. 8u+7 of
+// those 64 in the order 0,2,1,3,4,6,5,7 (what the two ANDs per dword leave in the 16-bit lanes).
+//
+// Data movement: a workgroup of 4 or 8 waves takes as many strips of 32 rows of W and a run of super-blocks.
+// Per super-block it needs the 16.5 KB of token operands (shared by its waves, converted from 16 KB of A) and
+// one 4.5 KB weight tile per wave, read from HBM in row-contiguous 144-byte runs straight into LDS
+// (global_load_lds_dwordx4) two super-blocks ahead of the arithmetic: a wave's weight tile is copied to
+// registers first and its LDS space is then the target of the tile after the next; the token operands
+// alternate between two LDS stages.  The weight tile lies in LDS row by row at a stride of 9 sixteen-byte pieces, which makes the
+// transposed reads (lane = row) conflict-free.  Two or three workgroups share a CU, so one workgroup's loads
+// overlap the others' arithmetic.  LDS is accessed through inline asm so that the compiler does not wait for
+// the loads in flight.
+#pragma once
+#include "kquant_common.hip.h"
+
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+namespace gemm_f16 {
+
+constexpr u32 kTokensPerTile = 16;
+constexpr u32 kMaxWaves = 8;                   // strips of 32 rows per workgroup: 4 or 8
+constexpr u32 kXpMainBytes = 16 * 1024;        // 16 products x 64 lanes x 16 bytes
+constexpr u32 kXpSumBytes = 512;               // 64 lanes x 4 f16
+constexpr u32 kXpFactorBytes = 64;             // 16 tokens x f32
+constexpr u32 kXpStageBytes = kXpMainBytes + kXpSumBytes + kXpFactorBytes;
+constexpr u32 kWStageBytes = 32 * 144;         // one super-block of 32 rows
+// dynamic LDS: two stages of token operands, two weight tiles per wave, one word for the arrival order
+__host__ __device__ constexpr u32 lds_bytes(u32 waves) { return 2u * kXpStageBytes + 2u * waves * kWStageBytes + 16u; }
+
+__device__ __forceinline__ u32 wave_max_u32(u32 v) {
+  v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true)));
+  v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, true)));
+  v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, true)));
+  v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, true)));
+  const u32 a = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(v), 0));
+  const u32 b = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(v), 16));
+  const u32 c = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(v), 32));
+  const u32 d = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(v), 48));
+  return max(max(a, b), max(c, d));
+}
+
+// hi and lo piece of a scaled value (|v| < 2^15, or not finite)
+__device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
+  hi = static_cast<_Float16>(v);
+  lo = static_cast<_Float16>((v - static_cast<float>(hi)) * 2048.0f);
+}
+
+__device__ __forceinline__ u32 pack_h2(_Float16 a, _Float16 b) {
+  const h16x2 p = {a, b};
+  return __builtin_bit_cast(u32, p);
+}
+
+// ---- LDS through inline asm ----------------------------------------------------------------------
+template <int OFF>
+__device__ __forceinline__ void lds_read128(u32x4& v, u32 addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read64(u32x2& v, u32 addr) {
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+// waits for every LDS read issued so far; the values pass through so that no use moves above the wait
+__device__ __forceinline__ void lds_wait4(u32x4& a, u32x4& b, u32x4& c, u32x4& d) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"memory");
+}
+__device__ __forceinline__ void lds_wait5(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e, u32x2& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f)::"memory");
+}
+
+__device__ __forceinline__ void dma16(const uint8_t* src, u32 lds_addr) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)(uintptr_t)lds_addr, 16, 0, 0);
+}
+
+__device__ __forceinline__ void lds_write128x2(u32 addr, const u32x4& a, const u32x4& b) {
+  asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16" ::"v"(addr), "v"(a), "v"(b) : "memory");
+}
+__device__ __forceinline__ void lds_write16x2(u32 addr, u32 a, u32 b) {     // the low halves of a and b, 8 bytes apart
+  asm volatile("ds_write_b16 %0, %1\n\tds_write_b16 %0, %2 offset:8" ::"v"(addr), "v"(a), "v"(b) : "memory");
+}
+__device__ __forceinline__ void lds_write32(u32 addr, u32 a) { asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(a) : "memory"); }
+
+// Token operands of one super-block, written to an LDS stage of kXpStageBytes:
+//   q*1024 + (32g + 2*token + piece)*16 + 2e   f16 = piece of the scaled element 32 j + 8 (u%4) + perm[e],
+//                                               u = q/2, h = q%2, j = 2 (2g + u/4) + h, perm = 0,2,1,3,4,6,5,7
+//   16384 + (32g + 2*token + piece)*8 + 2e     f16 = piece of 2^-5 * (sum of the scaled sub-block 4g + e)
+//   16896 + token*4                            f32 = 2^(E+14) where the run was scaled by 2^-E (NaN if the run
+//                                               holds an infinity or a NaN)
+// This thread brings the eight elements 8c .. 8c+7 (v0, v1) of token `token` of the tile; the 32 threads of a
+// half wave hold one token's run.
+__device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, u32 token, u32 c, u32 stage) {
+  const u32 lane = threadIdx.x & 63u;
+  const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+  u32 amax = 0u;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = max(amax, __float_as_uint(x[e]) & 0x7FFFFFFFu);
+  amax = max(amax, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(amax), 0xB1, 0xF, 0xF, true)));
+  amax = max(amax, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(amax), 0x4E, 0xF, 0xF, true)));
+  amax = max(amax, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(amax), 0x141, 0xF, 0xF, true)));
+  amax = max(amax, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(amax), 0x140, 0xF, 0xF, true)));
+  const u32 r0 = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(amax), 0));
+  const u32 r1 = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(amax), 16));
+  const u32 r2 = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(amax), 32));
+  const u32 r3 = static_cast<u32>(__builtin_amdgcn_readlane(static_cast<int>(amax), 48));
+  amax = lane < 32u ? max(r0, r1) : max(r2, r3);
+  u32 eb = amax >> 23;                      // biased exponent of the run's maximum
+  const bool finite = eb != 255u;
+  eb = eb < 14u ? 14u : eb;                 // keeps both powers of two normal; a run that tiny loses nothing that matters
+  const float down = __uint_as_float((268u - eb) << 23);        // 2^-E = 2^(141 - eb)
+  _Float16 hi[8], lo[8];
+  float xs[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    xs[e] = x[e] * down;
+    split_f16(xs[e], hi[e], lo[e]);
+  }
+  const u32 j = c >> 2, g = j >> 2, h = j & 1u, u = 4u * ((j & 3u) >> 1) + (c & 3u), q = 2u * u + h;
+  const u32x4 ph = {pack_h2(hi[0], hi[2]), pack_h2(hi[1], hi[3]), pack_h2(hi[4], hi[6]), pack_h2(hi[5], hi[7])};
+  const u32x4 pl = {pack_h2(lo[0], lo[2]), pack_h2(lo[1], lo[3]), pack_h2(lo[4], lo[6]), pack_h2(lo[5], lo[7])};
+  lds_write128x2(stage + q * 1024u + (32u * g + 2u * token) * 16u, ph, pl);
+  float sj = ((xs[0] + xs[1]) + (xs[2] + xs[3])) + ((xs[4] + xs[5]) + (xs[6] + xs[7]));
+  sj += dpp_f32<0xB1>(sj);
+  sj += dpp_f32<0x4E>(sj);                  // the four threads of a sub-block hold its sum
+  if ((c & 3u) == 0u) {
+    _Float16 sh, sl;
+    split_f16(sj * 0.03125f, sh, sl);
+    lds_write16x2(stage + kXpMainBytes + (32u * g + 2u * token) * 8u + 2u * (j & 3u), pack_h2(sh, sh), pack_h2(sl, sl));
+  }
+  if (c == 0u) lds_write32(stage + kXpMainBytes + kXpSumBytes + 4u * token, finite ? (eb << 23) : 0x7FC00000u);
+}
+
+__device__ __forceinline__ h16x2 pk_mul_h2(u32 bits, h16x2 s) { return as_h16x2(bits) * s; }
+
+// Main kernel.  Workgroup id -> (unit, token tile) with the token tiles of a unit 8 ids apart (same XCD, so the
+// weights they share meet in that XCD's L2); unit -> (group of 8 strips, part of K).  With one part the result
+// is stored; otherwise every part stores its partial result in `partial`, and the workgroup that arrives last
+// at the (group, tile) counter adds the parts in part order - the sum does not depend on who is last - and
+// puts the counter back to zero (the counters start at zero when the workspace is allocated).
+//   dynamic LDS = kLdsBytes
+template <int CHUNKS>     // chunks of A a thread converts per super-block: 512 / threads
+__device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
+                                         u32* __restrict__ counters, u32 m, u32 n, u32 nsb, u32 ksb, u32 kparts,
+                                         u32 groups, u32 tiles, u32 lds_base) {
+  const u32 lane = threadIdx.x & 63u;
+  const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
+  const u32 id = blockIdx.x;
+  const u32 unit = (id / (8u * tiles)) * 8u + (id & 7u), tile = (id >> 3) % tiles;
+  if (unit >= groups * kparts) return;
+  const u32 group = unit / kparts, part = unit - group * kparts;
+  const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
+  const u32 waves = blockDim.x >> 6;
+  const u32 strip = group * waves + wave;
+  const u32 col = lane & 31u, g = lane >> 5;
+  const size_t row_bytes = static_cast<size_t>(nsb) * 144u;
+
+  // where this lane's pieces of a weight tile come from: piece p = 64 t + lane of [32 rows][9 pieces]
+  size_t woff[5];
+#pragma unroll
+  for (int t = 0; t < 5; ++t) {
+    const u32 p = min(64u * t + lane, 287u);
+    const u32 r = p / 9u, cc = p - 9u * r;
+    woff[t] = static_cast<size_t>(min(strip * 32u + r, n - 1u)) * row_bytes + 16u * cc;
+  }
+  const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * (2u * kWStageBytes);
+  const u32 lds_flag = lds_base + 2u * kXpStageBytes + 2u * waves * kWStageBytes;
+  // the chunks of A this thread converts per super-block: 512 chunks of 8 elements (16 tokens x 32)
+  const u32 nthreads = blockDim.x;
+  const float* asrc[CHUNKS];
+  u32 ctoken[CHUNKS], cpos[CHUNKS];
+  bool live[CHUNKS];
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) {
+    const u32 idx = threadIdx.x + i * nthreads;
+    ctoken[i] = (idx >> 5) & 15u;
+    cpos[i] = idx & 31u;
+    const u32 token = tile * kTokensPerTile + ctoken[i];
+    asrc[i] = a + static_cast<size_t>(min(token, m - 1u)) * (static_cast<size_t>(nsb) * 256u) + 8u * cpos[i];
+    live[i] = token < m;
+  }
+
+  // Loads are counted by hand (s_waitcnt vmcnt): per super-block a wave issues 2*CHUNKS loads of A, then 5 of W.
+  auto issue_w = [&](u32 s) {
+    const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * 144u;
+    const u32 wl = lds_w + (s & 1u) * kWStageBytes;
+    dma16(wsrc + woff[0], wl);
+    dma16(wsrc + woff[1], wl + 1024u);
+    dma16(wsrc + woff[2], wl + 2048u);
+    dma16(wsrc + woff[3], wl + 3072u);
+    if (lane < 32u) dma16(wsrc + woff[4], wl + 4096u);
+  };
+  u32x4 an[CHUNKS][2];                 // A of a super-block on its way to conversion
+  auto load_a = [&](u32 s) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const float* src = asrc[i] + static_cast<size_t>(sb0 + s) * 256u;
+      asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
+                   : "=&v"(an[i][0]), "=&v"(an[i][1]) : "v"(src) : "memory");
+    }
+  };
+  auto convert = [&](u32 s) {          // the loads of A issued last have landed when 5 loads (of W) are left
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) asm volatile("s_waitcnt vmcnt(5)" : "+v"(an[i][0]), "+v"(an[i][1])::"memory");
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i)
+      convert_chunk(live[i] ? __builtin_bit_cast(f32x4, an[i][0]) : zero4, live[i] ? __builtin_bit_cast(f32x4, an[i][1]) : zero4,
+                    ctoken[i], cpos[i], lds_xp + (s & 1u) * kXpStageBytes);
+  };
+
+  f32x16 tot;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) tot[v] = 0.0f;
+
+  load_a(0);
+  issue_w(0);
+  convert(0);
+  if (ns > 1u) {
+    load_a(1);
+    issue_w(1);
+  }
+  for (u32 s = 0; s < ns; ++s) {
+    // weight tile s has landed (the loads of super-block s+1 may be in flight); the token operands of s are written
+    if (s + 1u < ns) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * CHUNKS + 5) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+    const u32 slot = s & 1u;
+    const u32 wt = lds_w + slot * kWStageBytes + col * 144u, wl = wt + g * 64u;
+    const u32 xl = lds_xp + slot * kXpStageBytes + lane * 16u;
+    const u32 sl = lds_xp + slot * kXpStageBytes + kXpMainBytes + lane * 8u;
+    const u32 fl = lds_xp + slot * kXpStageBytes + kXpMainBytes + kXpSumBytes + g * 8u;
+    u32x4 hdr, d0, d1, d2, d3;
+    u32x2 sx, f01, f23, f45, f67;
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(hdr) : "v"(wt) : "memory");
+    lds_read128<16>(d0, wl);
+    lds_read128<32>(d1, wl);
+    lds_read128<48>(d2, wl);
+    lds_read128<64>(d3, wl);
+    lds_read64<0>(sx, sl);
+    lds_read64<0>(f01, fl);          // 2^(E+14) of the tokens 4a + 2g + {0, 1}, a = 0..3
+    lds_read64<16>(f23, fl);
+    lds_read64<32>(f45, fl);
+    lds_read64<48>(f67, fl);
+    lds_wait5(hdr, d0, d1, d2, d3, sx);
+    asm volatile("" : "+v"(f01), "+v"(f23), "+v"(f45), "+v"(f67));
+    if (s + 1u < ns) convert(s + 1u);        // into the stage that was read two super-blocks ago
+    if (s + 2u < ns) {          // the weight tile is in registers: its LDS space takes the tile after the next
+      load_a(s + 2u);
+      issue_w(s + 2u);
+    }
+    const u32 dw[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w, d2.x, d2.y, d2.z, d2.w, d3.x, d3.y, d3.z, d3.w};
+    const float d = half_bits_to_f32(hdr.x), dmin = half_bits_to_f32(hdr.x >> 16);
+    // this lane's four 6-bit scales and mins as bytes (get_scale_min_k4, quantize.rs:1306-1385)
+    const u32 s4 = g ? ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u)) : (hdr.y & 0x3F3F3F3Fu);
+    const u32 m4 = g ? (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u)) : (hdr.z & 0x3F3F3F3Fu);
+    h16x2 sc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const _Float16 sv = static_cast<_Float16>(static_cast<unsigned short>((s4 >> (8 * e)) & 0xFFu)) *
+                          static_cast<_Float16>((e & 1) ? 64.0f : 1024.0f);
+      sc[e] = h16x2{sv, sv};
+    }
+    const h16x4 mb = {static_cast<_Float16>(static_cast<unsigned short>(m4 & 0xFFu)),
+                      static_cast<_Float16>(static_cast<unsigned short>((m4 >> 8) & 0xFFu)),
+                      static_cast<_Float16>(static_cast<unsigned short>((m4 >> 16) & 0xFFu)),
+                      static_cast<_Float16>(static_cast<unsigned short>(m4 >> 24))};
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const f32x16 macc = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx), mb, zero, 0, 0, 0);
+    f32x16 acc = zero;
+#pragma unroll
+    for (int uu = 0; uu < 8; uu += 2) {          // two dword pairs = four products per round of operand reads
+      u32x4 a0, a1, a2, a3;
+      switch (uu) {
+        case 0: lds_read128<0 * 1024>(a0, xl); lds_read128<1 * 1024>(a1, xl); lds_read128<2 * 1024>(a2, xl); lds_read128<3 * 1024>(a3, xl); break;
+        case 2: lds_read128<4 * 1024>(a0, xl); lds_read128<5 * 1024>(a1, xl); lds_read128<6 * 1024>(a2, xl); lds_read128<7 * 1024>(a3, xl); break;
+        case 4: lds_read128<8 * 1024>(a0, xl); lds_read128<9 * 1024>(a1, xl); lds_read128<10 * 1024>(a2, xl); lds_read128<11 * 1024>(a3, xl); break;
+        default: lds_read128<12 * 1024>(a0, xl); lds_read128<13 * 1024>(a1, xl); lds_read128<14 * 1024>(a2, xl); lds_read128<15 * 1024>(a3, xl); break;
+      }
+      const u32x4* aq[4] = {&a0, &a1, &a2, &a3};
+      u32 bl[2][4], bh[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int u = uu + i;
+        const u32 t0 = dw[2 * u], t1 = dw[2 * u + 1], t0s = t0 >> 8, t1s = t1 >> 8;
+        const h16x2 sl2 = sc[(u >> 2) * 2], sh2 = sc[(u >> 2) * 2 + 1];
+        bl[i][0] = __builtin_bit_cast(u32, pk_mul_h2(t0 & 0x000F000Fu, sl2));
+        bl[i][1] = __builtin_bit_cast(u32, pk_mul_h2(t0s & 0x000F000Fu, sl2));
+        bl[i][2] = __builtin_bit_cast(u32, pk_mul_h2(t1 & 0x000F000Fu, sl2));
+        bl[i][3] = __builtin_bit_cast(u32, pk_mul_h2(t1s & 0x000F000Fu, sl2));
+        bh[i][0] = __builtin_bit_cast(u32, pk_mul_h2(t0 & 0x00F000F0u, sh2));
+        bh[i][1] = __builtin_bit_cast(u32, pk_mul_h2(t0s & 0x00F000F0u, sh2));
+        bh[i][2] = __builtin_bit_cast(u32, pk_mul_h2(t1 & 0x00F000F0u, sh2));
+        bh[i][3] = __builtin_bit_cast(u32, pk_mul_h2(t1s & 0x00F000F0u, sh2));
+      }
+      lds_wait4(a0, a1, a2, a3);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const u32x4 blv = {bl[i][0], bl[i][1], bl[i][2], bl[i][3]}, bhv = {bh[i][0], bh[i][1], bh[i][2], bh[i][3]};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[2 * i]), __builtin_bit_cast(h16x8, blv), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[2 * i + 1]), __builtin_bit_cast(h16x8, bhv), acc, 0, 0, 0);
+      }
+    }
+    const float nm = dmin * -0.001953125f;       // -dmin * 2^-9: the sums carry 2^-5, the products 2^-14
+    const float fac[8] = {__uint_as_float(f01.x), __uint_as_float(f01.y), __uint_as_float(f23.x), __uint_as_float(f23.y),
+                          __uint_as_float(f45.x), __uint_as_float(f45.y), __uint_as_float(f67.x), __uint_as_float(f67.y)};
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float fd = fac[t] * d, fm = fac[t] * nm;
+      tot[2 * t] = fmaf(fm, macc[2 * t], fmaf(fd, acc[2 * t], tot[2 * t]));
+      tot[2 * t + 1] = fmaf(fm, macc[2 * t + 1], fmaf(fd, acc[2 * t + 1], tot[2 * t + 1]));
+    }
+  }
+
+  // lane l, registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row strip*32 + col
+  const u32 row = strip * 32u + col;
+  const bool row_ok = row < n;
+  const u32 tokens_pad = tiles * kTokensPerTile;
+  float val[8];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) val[2 * a + b] = fmaf(tot[4 * a + 2 * b + 1], 0.00048828125f, tot[4 * a + 2 * b]);
+  if (kparts == 1u) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
+        if (row_ok && token < m) c[static_cast<size_t>(token) * n + row] = val[2 * a + b];
+      }
+    return;
+  }
+  // several parts of K: publish this part, the last arrival adds them up
+  if (row_ok)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
+        if (token < m)
+          __hip_atomic_store(reinterpret_cast<u32*>(partial) + (static_cast<size_t>(part) * tokens_pad + token) * n + row,
+                             __float_as_uint(val[2 * a + b]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
+  asm volatile("s_barrier" ::: "memory");
+  if (threadIdx.x == 0u) {
+    const u32 old = __hip_atomic_fetch_add(counters + group * tiles + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(lds_flag), "v"(old) : "memory");
+  }
+  asm volatile("s_barrier" ::: "memory");
+  u32 old;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(lds_flag) : "memory");
+  if (old == kparts - 1u && threadIdx.x == 0u)      // ready for the next product on this stream
+    __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (old != kparts - 1u || !row_ok) return;
+  float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // up to 64 loads in flight, added in part order
+    u32 got[8][8];
+#pragma unroll
+    for (int pp = 0; pp < 8; ++pp)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
+        got[pp][t] = 0u;
+        if (p0 + pp < kparts && token < m)
+          got[pp][t] = __hip_atomic_load(reinterpret_cast<const u32*>(partial) + (static_cast<size_t>(p0 + pp) * tokens_pad + token) * n + row,
+                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+    for (int pp = 0; pp < 8; ++pp)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) r[t] += __uint_as_float(got[pp][t]);
+  }
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
+    if (token < m) c[static_cast<size_t>(token) * n + row] = r[t];
+  }
+}
+
+}  // namespace gemm_f16

@@ -10,7 +10,7 @@
 // multiple of 64.
 #include "kquant_chain.hip.h"
 #include "kquant_stream.hip.h"
-#include "kquant_gemm_mfma.hip.h"
+#include "kquant_gemm_f16.hip.h"
 
 // The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
 // activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
@@ -147,21 +147,19 @@ KQ_GEMM_KERNELS(q4k, FMT_Q4K)
 KQ_GEMM_KERNELS(q5k, FMT_Q5K)
 KQ_GEMM_KERNELS(q6k, FMT_Q6K)
 
-// Matrix-core form of the Q4_K GEMM for m >= 2 (kquant_gemm_mfma.hip.h): digit planes of A, then the product.
-extern "C" __global__ void __launch_bounds__(256)
-kq_gemm_planes(const float* a, uint8_t* planes, float* meta, float* c, u32 m, u32 n, u32 k, u32 clear_c) {
-  gemm_mfma::planes_body(a, planes, meta, c, m, n, k, clear_c);
-}
-extern "C" __global__ void __launch_bounds__(256)
-q4k_gemm_mfma_t1(const uint8_t* planes, const float* meta, const uint8_t* w, float* c, u32 m, u32 n, u32 k) {
-  gemm_mfma::q4k_body<1>(planes, meta, w, c, m, n, k);
-}
-extern "C" __global__ void __launch_bounds__(256)
-q4k_gemm_mfma_t2(const uint8_t* planes, const float* meta, const uint8_t* w, float* c, u32 m, u32 n, u32 k) {
-  gemm_mfma::q4k_body<2>(planes, meta, w, c, m, n, k);
-}
+// Matrix-core form of the Q4_K GEMM for m >= 2 (kquant_gemm_f16.hip.h).
+#define KQ_GEMM_F16(name, threads)                                                                                      \
+  extern "C" __global__ void __launch_bounds__(threads)                                                                  \
+  name(const float* a, const uint8_t* w, float* c, float* partial, u32* counters, u32 m, u32 n, u32 nsb, u32 ksb,        \
+       u32 kparts, u32 groups, u32 tiles) {                                                                              \
+    extern __shared__ uint8_t gemm_lds[];                                                                                \
+    const u32 lds_base =                                                                                                 \
+        static_cast<u32>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) uint8_t*)gemm_lds));         \
+    gemm_f16::q4k_body<512 / threads>(a, w, c, partial, counters, m, n, nsb, ksb, kparts, groups, tiles, lds_base);      \
+  }
+KQ_GEMM_F16(q4k_gemm_f16_w8, 512)
+KQ_GEMM_F16(q4k_gemm_f16_w4, 256)
 
-// ------------------------------------------------------------------------------------------
 // Legacy "simplified" Q4_K (trueno-gpu/src/kernels/quantize.rs:151-336, kernel name q4k_gemm_fused): blocks of 32
 // values in 18 bytes - f16 scale at 0, 16 bytes of nibbles at 2, value i in byte i/2 (low nibble for even i);
 // w = scale * q, no min term (:237-267).  W is n rows x k/32 blocks, row-major (:225-231); the product is the

@@ -65,7 +65,7 @@ struct DeviceKernels {
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
-  hipFunction_t gemm_planes = nullptr, gemm_mfma[2] = {};
+  hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
@@ -78,9 +78,8 @@ int g_tune_chain_spin_limit = 0;
 int g_tune_stream_consumers = 0;
 int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
-int g_tune_gemm_tiles = 0;      // token tiles (of 8) per wave in the matrix-core GEMM: 1 or 2
-int g_tune_gemm_ksplit = 0;     // parts of K per row tile: 1 or 2
-int g_tune_gemm_waves = 0;      // waves per workgroup of the matrix-core GEMM: 1..4   // 1: never fuse independent GEMVs of a list into one launch
+int g_tune_gemm_ksplit = 0;     // parts of K in the matrix-core GEMM (0: chosen from the shape)
+int g_tune_gemm_waves = 0;      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -124,11 +123,10 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
         (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
-        (e = get_fn(m, &t.gemm_planes, "kq_gemm_planes")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
         (e = get_fn(m, &t.dequant_simplified, "q4k_simplified_dequant_f32")) != hipSuccess ||
-        (e = get_fn(m, &t.gemm_mfma[0], "q4k_gemm_mfma_t1")) != hipSuccess ||
-        (e = get_fn(m, &t.gemm_mfma[1], "q4k_gemm_mfma_t2")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[0], "q4k_gemm_f16_w4")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[1], "q4k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -194,17 +192,32 @@ bool gemv_fast_ok(Fmt f, uint64_t y, uint64_t w, uint64_t x) {
   return aligned(x, 16) && aligned(y, 4) && aligned(w, f == Q6K ? 2 : 16);
 }
 
-// Digit planes of A for the matrix-core GEMM: one buffer per (device, stream), grown on demand and kept.
+// Partial results and arrival counters of the matrix-core GEMM: one buffer per (device, stream), grown on
+// demand and kept.  The counters are zero between products: the kernel puts them back.
 struct GemmWorkspace {
-  void* planes = nullptr;
+  void* buf = nullptr;
   size_t cap = 0;
 };
 std::map<std::pair<int, hipStream_t>, GemmWorkspace> g_gemm_ws;
 
-hipError_t launch_q4k_gemm_mfma(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
-                                uint32_t n, uint32_t k) {
-  const uint32_t nsb = k / 256u, tiles = (m + 7u) / 8u;
-  const size_t planes_bytes = size_t(tiles) * nsb * 8192u, meta_bytes = size_t(tiles) * nsb * 72u * 4u;
+constexpr uint32_t kGemmXpStageBytes = 16 * 1024 + 512 + 64, kGemmWTileBytes = 32 * 144;
+
+hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
+                               uint32_t n, uint32_t k) {
+  const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
+  // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
+  const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
+  const uint32_t lds = 2u * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
+  const uint32_t groups = (n + 32u * waves - 1u) / (32u * waves);
+  // cut K so that the workgroups are about as many as the CUs
+  const uint64_t units = uint64_t(groups) * tiles;
+  uint32_t kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d->cu_count) + units / 2u) / units);
+  kparts = std::min(std::max(kparts, 1u), nsb);
+  const uint32_t ksb = (nsb + kparts - 1u) / kparts;
+  kparts = (nsb + ksb - 1u) / ksb;
+  auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
+  const size_t cnt_bytes = up(size_t(groups) * tiles * 4u);
+  const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * 16u * n * 4u) : 0u;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
@@ -213,32 +226,25 @@ hipError_t launch_q4k_gemm_mfma(DeviceKernels* d, hipStream_t stream, uint64_t a
     std::lock_guard<std::mutex> lock(g_mutex);
     ws = &g_gemm_ws[std::make_pair(dev, stream)];
   }
-  if (ws->cap < planes_bytes + meta_bytes) {
-    if (ws->planes) {
-      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;   // a GEMM in flight may still read it
-      (void)hipFree(ws->planes);
-      ws->planes = nullptr;
+  // the counters sit at the end of a region that only grows, so a larger product finds zeros there too
+  const size_t cnt_cap = up(size_t(1) << 16), need = cnt_cap + part_bytes;
+  if (cnt_bytes > cnt_cap) return hipErrorInvalidValue;
+  if (ws->cap < need) {
+    if (ws->buf) {
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;   // a GEMM in flight may still use it
+      (void)hipFree(ws->buf);
+      ws->buf = nullptr;
       ws->cap = 0;
     }
-    if ((e = hipMalloc(&ws->planes, planes_bytes + meta_bytes)) != hipSuccess) return e;
-    ws->cap = planes_bytes + meta_bytes;
+    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
+    ws->cap = need;
+    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;
   }
-  uint64_t planes = reinterpret_cast<uint64_t>(ws->planes), meta = planes + planes_bytes;
-  uint32_t t = g_tune_gemm_tiles > 0 ? uint32_t(g_tune_gemm_tiles) : 1u;   // measured: two tiles per wave never pay
-  t = std::min(std::max(t, 1u), 2u);
-  const uint32_t gx = (n + 31u) / 32u, gy = (tiles + t - 1u) / t;
-  uint32_t ksplit = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : (uint64_t(gx) * gy < uint64_t(d->cu_count) * 8u ? 2u : 1u);
-  ksplit = std::min(std::min(std::max(ksplit, 1u), 2u), nsb);
-  uint32_t clear_c = ksplit > 1 ? 1u : 0u;
-  void* pargs[] = {&a, &planes, &meta, &c, &m, &n, &k, &clear_c};
-  const uint64_t items = uint64_t(tiles) * 8u * nsb;
-  const uint32_t pgrid = uint32_t(std::min<uint64_t>((items + 3) / 4, uint64_t(d->cu_count) * 16u));
-  if ((e = hipModuleLaunchKernel(d->gemm_planes, pgrid, 1, 1, 256, 1, 1, 0, stream, pargs, nullptr)) != hipSuccess) return e;
-  void* margs[] = {&planes, &meta, &w, &c, &m, &n, &k};
-  // waves of a workgroup share a part of K: as many as leave each at least two super-blocks, four at most
-  uint32_t waves = g_tune_gemm_waves > 0 ? uint32_t(g_tune_gemm_waves) : 4u;
-  waves = std::max(1u, std::min(std::min(waves, 4u), std::max(1u, nsb / ksplit / 2u)));
-  return hipModuleLaunchKernel(d->gemm_mfma[t - 1], gx, gy, ksplit, 64 * waves, 1, 1, 0, stream, margs, nullptr);
+  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
+  uint32_t nsb_arg = nsb, ksb_arg = ksb, kparts_arg = kparts, groups_arg = groups, tiles_arg = tiles;
+  void* margs[] = {&a, &w, &c, &part, &cnt, &m, &n, &nsb_arg, &ksb_arg, &kparts_arg, &groups_arg, &tiles_arg};
+  return hipModuleLaunchKernel(d->gemm_f16[waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
@@ -250,8 +256,8 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
   if (!is_gemv && f == Q4K && m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
-      (n + 31u) / 32u <= 65535u * 32u && (m + 7u) / 8u <= 65535u)
-    return launch_q4k_gemm_mfma(d, stream, a, w, c, m, n, k);
+      uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u)   // its arrival counters
+    return launch_q4k_gemm_f16(d, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
@@ -1044,7 +1050,6 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "gemm_tiles_per_wave")) { g_tune_gemm_tiles = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
