@@ -120,6 +120,9 @@ def main() -> int:
         wbytes += HEAD[2] * (HEAD[3] // 256) * SB[HEAD[1]]
         return b, nbytes, wbytes
 
+    for kv in filter(None, os.environ.get("TRN_BENCH_TUNE", "").split(",")):      # working aid: library tuning keys
+        key, val = kv.split("=")
+        assert L.trn_set_tuning(key.encode(), int(val)) == 0, kv
     batch, total_bytes, weight_bytes = build_pass(False)
     strict_batch, _, _ = build_pass(True)
 

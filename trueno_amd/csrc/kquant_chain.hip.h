@@ -28,12 +28,9 @@
 #pragma once
 #include "kquant_quarter.hip.h"
 
-#ifdef CHAIN_TS
-extern __device__ unsigned long long* g_chain_ts;   // [entry][8] for workgroup CHAIN_TS_WG: 0 start, 1 after wait, 2 after x, 3 end, 4 after sum of squares, 5 after row loop
-#define CHAIN_STAMP(slot) do { if (g_chain_ts && blockIdx.x == g_chain_ts_wg && threadIdx.x == 0) g_chain_ts[8 * g_chain_ts_entry + (slot)] = wall_clock64(); } while (0)
-extern __device__ unsigned g_chain_ts_wg;
-static __device__ unsigned g_chain_ts_entry;
-#else
+// CHAIN_STAMP(slot): a hook for timing probes (0 start, 1 after the barrier wait, 2 activations staged, 4 after the
+// sum of squares, 5 after the row loop, 3 end); a probe defines it before including this file.
+#ifndef CHAIN_STAMP
 #define CHAIN_STAMP(slot) do { } while (0)
 #endif
 
