@@ -279,6 +279,26 @@ def main() -> int:
             for b in bufs:
                 b.free()
 
+    # ---- the element-wise steps between the GEMVs of a layer, one launch each (latency-bound: a few KB) ----------
+    glue_us = {}
+    if not args.no_configs:
+        hid, ffn = 4096, 11008
+        g_a, g_b, g_o, g_g = (t.GpuBuffer.from_host(ctx, kq.gen_x(9000 + i, ffn)) for i in range(4))
+        for label, fn in (("residual_add_4096", lambda: L.trn_residual_add(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), hid)),
+                          ("rmsnorm_4096", lambda: L.trn_rmsnorm(stream.raw(), g_a.as_ptr(), g_o.as_ptr(), g_g.as_ptr(), hid, C.c_float(1e-5))),
+                          ("fused_residual_rmsnorm_4096", lambda: L.trn_fused_residual_rmsnorm(
+                              stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), g_g.as_ptr(), hid, C.c_float(1e-5))),
+                          ("fused_swiglu_11008", lambda: L.trn_fused_swiglu(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), ffn))):
+            for _ in range(8):
+                fn()
+            stream.synchronize()
+            L.trn_event_record(e0, stream.raw())
+            for _ in range(64):
+                fn()
+            L.trn_event_record(e1, stream.raw())
+            stream.synchronize()
+            glue_us[label] = round(elapsed_ms(e0, e1) * 1e3 / 64, 2)
+
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
     cpu_config1 = None
@@ -332,7 +352,7 @@ def main() -> int:
                   "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
                   "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
-                  "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes,
+                  "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }

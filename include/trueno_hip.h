@@ -168,6 +168,23 @@ TRN_API trn_status trn_event_destroy(trn_event event);
 TRN_API trn_status trn_event_record(trn_event event, trn_stream stream);
 TRN_API trn_status trn_event_synchronize(trn_event event);
 TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop);
+/* ---- element-wise steps between the GEMVs of a decoder layer (f32 vectors) ---------------------------------
+ * The same kernels are in the built-in module under the reference's names "residual_add", "fused_swiglu",
+ * "rmsnorm", "fused_residual_rmsnorm".  The first two keep the reference's parameter lists; the reference
+ * compiles hidden_size and epsilon of the two norms into its PTX, here they follow the pointers as two more
+ * parameters (u32 hidden_size, f32 epsilon).  Whatever grid and block a by-name launch passes is replaced. */
+/* output[i] = input1[i] + input2[i]; output may alias an input.  trueno-gpu/src/kernels/elementwise.rs:33-101 */
+TRN_API trn_status trn_residual_add(trn_stream stream, trn_dptr input1, trn_dptr input2, trn_dptr output, uint32_t n);
+/* output[i] = silu(gate[i]) * up[i], silu(g) = g / (1 + 2^(-g * 1.442695f)).  elementwise.rs:521-592 */
+TRN_API trn_status trn_fused_swiglu(trn_stream stream, trn_dptr gate, trn_dptr up, trn_dptr output, uint32_t n);
+/* One row: output[i] = input[i] * rsqrt(mean(input^2) + epsilon) * gamma[i]; output may alias input.
+ * trueno-gpu/src/kernels/layernorm.rs:388-516 (RmsNormKernel; its default epsilon is 1e-5, :400-405) */
+TRN_API trn_status trn_rmsnorm(trn_stream stream, trn_dptr input, trn_dptr output, trn_dptr gamma, uint32_t hidden_size,
+                               float epsilon);
+/* One row: the same with x = residual + input; output may alias residual.  elementwise.rs:109-248 */
+TRN_API trn_status trn_fused_residual_rmsnorm(trn_stream stream, trn_dptr residual, trn_dptr input, trn_dptr output,
+                                              trn_dptr gamma, uint32_t hidden_size, float epsilon);
+
 /* dst[0..bytes) = src[0..bytes) with one 16-byte load and store per lane; bytes % 16 == 0.
  * The plain-copy yardstick that HBM counters are scaled by. */
 TRN_API trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t bytes);

@@ -1,0 +1,93 @@
+"""CPU oracle for the element-wise decoder-layer kernels (TEST INFRASTRUCTURE ONLY).
+
+A numpy restatement of the instruction sequences trueno-gpu's PTX builder describes; only tests/,
+__graft_entry__.smoke() and bench.py may import it.
+
+Reference lines followed (under trueno-gpu/src/kernels/):
+  residual_add            elementwise.rs:33-101    add.f32
+  fused_swiglu            elementwise.rs:521-592   sub, mul by 1.442695f, ex2.approx, add, div.rn, mul, mul
+  rmsnorm                 layernorm.rs:388-516     32 lanes, fma per element, shfl.down tree, div.rn, add, rsqrt.approx, mul, mul
+  fused_residual_rmsnorm  elementwise.rs:109-248   the same on x = residual + input
+(div.f32 is printed as div.rn, ex2/rsqrt as .approx: trueno-gpu/src/ptx/builder.rs:1425-1431, 1523-1530.)
+
+Every f32 operation is rounded separately, as the reference's instructions are.  The two approximate
+instructions are evaluated exactly here (fp64, rounded to f32); PTX documents them to 2^-22 relative, so the
+reference's own outputs lie within that of this oracle, and so must any implementation - that is the tolerance
+the tests state.
+
+How each function is pinned (the reference holds no numeric test of these kernels, only names and PTX text):
+  residual_add          : exact by definition.
+  fused_swiglu          : closed forms (gate = 0 -> 0; large gate -> gate*up; silu(g) - silu(-g) = g), agreement with
+                          the fp64 formula gate/(1+exp(-gate))*up (the f32 constant 1.442695 is not log2(e) to the last
+                          bit: the difference is covered and bounded in the tests).
+  rmsnorm*              : closed forms (constant rows, one-hot rows), mean square of the output, scale invariance,
+                          agreement with the fp64 formula; the lane order is an emulation used for error magnitudes.
+Against a running reference these stay "parity unpinned": it cannot be run here (no Rust, no NVIDIA driver).
+"""
+import numpy as np
+
+F32 = np.float32
+LOG2E_F32 = F32(1.442695)          # the literal of elementwise.rs:570
+
+
+def residual_add(a, b):
+    return (np.asarray(a, F32) + np.asarray(b, F32)).astype(F32)
+
+
+def fused_swiglu(gate, up):
+    """elementwise.rs:565-582, one rounding per instruction, ex2 exact."""
+    g = np.asarray(gate, F32)
+    u = np.asarray(up, F32)
+    neg = (F32(0.0) - g).astype(F32)
+    scaled = (neg * LOG2E_F32).astype(F32)
+    with np.errstate(over="ignore", under="ignore"):
+        e = np.exp2(scaled.astype(np.float64)).astype(F32)
+        denom = (F32(1.0) + e).astype(F32)
+        sigmoid = (F32(1.0) / denom).astype(F32)
+    silu = (g * sigmoid).astype(F32)
+    return (silu * u).astype(F32)
+
+
+def fused_swiglu_fp64(gate, up):
+    g = np.asarray(gate, np.float64)
+    with np.errstate(over="ignore"):
+        return g / (1.0 + np.exp(-g)) * np.asarray(up, np.float64)
+
+
+def _fma32(a, b, c):
+    """fma.rn.f32: the product of two f32 is exact in f64; one further rounding error of 2^-53 relative is far below f32's."""
+    return F32(np.float64(a) * np.float64(b) + np.float64(c))
+
+
+def sum_squares_ref_order(x):
+    """layernorm.rs:441-474: lane t of 32 takes elements t, t+32, ... by fma; then shfl.down 16, 8, 4, 2, 1."""
+    x = np.asarray(x, F32)
+    lanes = np.zeros(32, F32)
+    for t in range(32):
+        acc = F32(0.0)
+        for v in x[t::32]:
+            acc = _fma32(v, v, acc)
+        lanes[t] = acc
+    for d in (16, 8, 4, 2, 1):
+        nxt = lanes.copy()
+        nxt[:32 - d] = (lanes[:32 - d] + lanes[d:]).astype(F32)
+        lanes = nxt
+    return lanes[0]
+
+
+def rmsnorm(x, gamma, eps=1e-5, residual=None):
+    """layernorm.rs:476-507 / elementwise.rs:212-240 with the exact reciprocal square root."""
+    x = np.asarray(x, F32)
+    if residual is not None:
+        x = (np.asarray(residual, F32) + x).astype(F32)
+    total = sum_squares_ref_order(x)
+    mean_sq = F32(total / F32(len(x)))
+    rms_inv = F32(1.0 / np.sqrt(np.float64(F32(mean_sq + F32(eps)))))
+    return ((x * rms_inv).astype(F32) * np.asarray(gamma, F32)).astype(F32)
+
+
+def rmsnorm_fp64(x, gamma, eps=1e-5, residual=None):
+    x = np.asarray(x, np.float64)
+    if residual is not None:
+        x = (np.asarray(residual, F32) + np.asarray(x, F32)).astype(np.float64)     # the add is an f32 add in the reference
+    return x / np.sqrt(np.mean(x * x) + np.float64(F32(eps))) * np.asarray(gamma, np.float64)

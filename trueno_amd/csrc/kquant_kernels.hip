@@ -11,6 +11,7 @@
 #include "kquant_chain.hip.h"
 #include "kquant_stream.hip.h"
 #include "kquant_gemm_f16.hip.h"
+#include "decode_glue.hip.h"
 
 // The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
 // activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
@@ -113,6 +114,27 @@ extern "C" __global__ void __launch_bounds__(512)
 kq_gemv_stream(const ChainEntry* entries, u32 count, u32* counters, u32* status, u32 spin_limit, u32 x_bytes_max,
                u32 rows_max, u32 slabs_max) {
   stream::stream_body(entries, count, counters, status, spin_limit, x_bytes_max, rows_max, slabs_max);
+}
+
+// ------------------------------------------------------------------------------------------
+// Element-wise steps of a decoder layer under the reference's kernel names (decode_glue.hip.h).  residual_add and
+// fused_swiglu keep the reference's parameter lists (elementwise.rs:56-59, 541-544).  The reference compiles the
+// row length and epsilon of rmsnorm / fused_residual_rmsnorm into the PTX (layernorm.rs:424-431,
+// elementwise.rs:145-149); with one pre-built code object they are two more parameters after the pointers.
+// ------------------------------------------------------------------------------------------
+extern "C" __global__ void __launch_bounds__(256) residual_add(const float* input1, const float* input2, float* output, u32 n) {
+  glue::residual_add_body(input1, input2, output, n);
+}
+extern "C" __global__ void __launch_bounds__(256) fused_swiglu(const float* gate, const float* up, float* output, u32 n) {
+  glue::fused_swiglu_body(gate, up, output, n);
+}
+extern "C" __global__ void __launch_bounds__(1024)
+rmsnorm(const float* input, float* output, const float* gamma, u32 hidden_size, float epsilon) {
+  glue::rmsnorm_body<false>(nullptr, input, output, gamma, hidden_size, epsilon);
+}
+extern "C" __global__ void __launch_bounds__(1024)
+fused_residual_rmsnorm(const float* residual, const float* input, float* output, const float* gamma, u32 hidden_size, float epsilon) {
+  glue::rmsnorm_body<true>(residual, input, output, gamma, hidden_size, epsilon);
 }
 
 extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32 v) {

@@ -43,7 +43,8 @@ const char* const kFmtName[NFMT] = {"q4k", "q5k", "q6k"};
 const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 
 // kinds of functions the launch-by-name path recognises
-enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3 };
+enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3, KIND_RESIDUAL_ADD = 4, KIND_SWIGLU = 5,
+            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7 };
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
@@ -65,6 +66,7 @@ struct DeviceKernels {
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
+  hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
@@ -120,6 +122,10 @@ hipError_t device_kernels(DeviceKernels** out) {
       }
     }
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
+        (e = get_fn(m, &t.residual_add, "residual_add")) != hipSuccess ||
+        (e = get_fn(m, &t.swiglu, "fused_swiglu")) != hipSuccess ||
+        (e = get_fn(m, &t.rmsnorm, "rmsnorm")) != hipSuccess ||
+        (e = get_fn(m, &t.residual_rmsnorm, "fused_residual_rmsnorm")) != hipSuccess ||
         (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
         (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
@@ -190,6 +196,37 @@ bool gemv_fast_ok(Fmt f, uint64_t y, uint64_t w, uint64_t x) {
   // 128-bit activation loads; Q4_K/Q5_K blocks are streamed with aligned 128-bit loads (their
   // rows are multiples of 16 bytes); Q6_K blocks (210 bytes) only need their natural 2 bytes.
   return aligned(x, 16) && aligned(y, 4) && aligned(w, f == Q6K ? 2 : 16);
+}
+
+// Element-wise steps of a decoder layer (decode_glue.hip.h).  kind: KIND_RESIDUAL_ADD or KIND_SWIGLU.
+hipError_t launch_elementwise(Kind kind, hipStream_t stream, uint64_t a, uint64_t b, uint64_t out, uint32_t n) {
+  if (n == 0) return hipSuccess;
+  if (!a || !b || !out || !aligned(a, 4) || !aligned(b, 4) || !aligned(out, 4)) return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  const uint32_t grid = std::max(1u, std::min((n + 255u) / 256u, uint32_t(d->cu_count) * 8u));
+  void* args[] = {&a, &b, &out, &n};
+  return hipModuleLaunchKernel(kind == KIND_SWIGLU ? d->swiglu : d->residual_add, grid, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
+}
+
+// residual == 0: rmsnorm; else fused_residual_rmsnorm.  One row, one workgroup.
+hipError_t launch_rmsnorm(hipStream_t stream, uint64_t residual, uint64_t in, uint64_t out, uint64_t gamma, uint32_t hidden,
+                          float eps, bool with_residual) {
+  if (hidden == 0) return hipSuccess;
+  if (!in || !out || !gamma || (with_residual && !residual) || !aligned(in, 4) || !aligned(out, 4) || !aligned(gamma, 4) ||
+      !aligned(residual, 4))
+    return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  const uint32_t block = hidden <= 256u ? 64u : hidden <= 2048u ? 256u : 1024u;
+  if (with_residual) {
+    void* args[] = {&residual, &in, &out, &gamma, &hidden, &eps};
+    return hipModuleLaunchKernel(d->residual_rmsnorm, 1, 1, 1, block, 1, 1, 0, stream, args, nullptr);
+  }
+  void* args[] = {&in, &out, &gamma, &hidden, &eps};
+  return hipModuleLaunchKernel(d->rmsnorm, 1, 1, 1, block, 1, 1, 0, stream, args, nullptr);
 }
 
 // Partial results and arrival counters of the matrix-core GEMM: one buffer per (device, stream), grown on
@@ -743,6 +780,10 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
       if (n == std::string(kFmtName[i]) + "_gemm_ggml") { h->kind = KIND_GEMM; h->fmt = i; }
     }
     if (n == "q4k_gemm_fused") h->kind = KIND_GEMM_SIMPLIFIED;
+    if (n == "residual_add") h->kind = KIND_RESIDUAL_ADD;
+    if (n == "fused_swiglu") h->kind = KIND_SWIGLU;
+    if (n == "rmsnorm") h->kind = KIND_RMSNORM;
+    if (n == "fused_residual_rmsnorm") h->kind = KIND_RESIDUAL_RMSNORM;
   }
   module->functions[name] = h;
   *func = h;
@@ -849,6 +890,30 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     if (func->kind == KIND_GEMM_SIMPLIFIED) return st(launch_gemm_simplified(s, p0, p1, p2, m, n, k));
     return st(launch_gemm_like(Fmt(func->fmt), s, p0, p1, p2, m, n, k, false));
   }
+  if (func->kind == KIND_RESIDUAL_ADD || func->kind == KIND_SWIGLU) {          // (ptr, ptr, output_ptr, n)
+    if (!kernel_params || !kernel_params[0] || !kernel_params[1] || !kernel_params[2] || !kernel_params[3]) return TRN_ERROR_INVALID_VALUE;
+    uint64_t p0, p1, p2;
+    uint32_t n;
+    std::memcpy(&p0, kernel_params[0], 8);
+    std::memcpy(&p1, kernel_params[1], 8);
+    std::memcpy(&p2, kernel_params[2], 8);
+    std::memcpy(&n, kernel_params[3], 4);
+    return st(launch_elementwise(Kind(func->kind), s, p0, p1, p2, n));
+  }
+  if (func->kind == KIND_RMSNORM || func->kind == KIND_RESIDUAL_RMSNORM) {     // pointers, then hidden_size, epsilon
+    const int np = func->kind == KIND_RMSNORM ? 3 : 4;
+    if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
+    for (int i = 0; i < np + 2; ++i)
+      if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
+    uint64_t p[4] = {0, 0, 0, 0};
+    for (int i = 0; i < np; ++i) std::memcpy(&p[i], kernel_params[i], 8);
+    uint32_t hidden;
+    float eps;
+    std::memcpy(&hidden, kernel_params[np], 4);
+    std::memcpy(&eps, kernel_params[np + 1], 4);
+    if (np == 3) return st(launch_rmsnorm(s, 0, p[0], p[1], p[2], hidden, eps, false));
+    return st(launch_rmsnorm(s, p[0], p[1], p[2], p[3], hidden, eps, true));
+  }
   return st(hipModuleLaunchKernel(func->fn, grid_x, grid_y, grid_z, block_x, block_y, block_z, shared_mem_bytes, s,
                                   kernel_params, extra));
 }
@@ -934,6 +999,20 @@ trn_status trn_q4k_gemm_fused(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dp
 
 trn_status trn_q4k_simplified_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w, uint64_t n_blocks) {
   return st(launch_dequant_simplified(static_cast<hipStream_t>(s), out, w, n_blocks));
+}
+
+trn_status trn_residual_add(trn_stream s, trn_dptr input1, trn_dptr input2, trn_dptr output, uint32_t n) {
+  return st(launch_elementwise(KIND_RESIDUAL_ADD, static_cast<hipStream_t>(s), input1, input2, output, n));
+}
+trn_status trn_fused_swiglu(trn_stream s, trn_dptr gate, trn_dptr up, trn_dptr output, uint32_t n) {
+  return st(launch_elementwise(KIND_SWIGLU, static_cast<hipStream_t>(s), gate, up, output, n));
+}
+trn_status trn_rmsnorm(trn_stream s, trn_dptr input, trn_dptr output, trn_dptr gamma, uint32_t hidden_size, float epsilon) {
+  return st(launch_rmsnorm(static_cast<hipStream_t>(s), 0, input, output, gamma, hidden_size, epsilon, false));
+}
+trn_status trn_fused_residual_rmsnorm(trn_stream s, trn_dptr residual, trn_dptr input, trn_dptr output, trn_dptr gamma,
+                                      uint32_t hidden_size, float epsilon) {
+  return st(launch_rmsnorm(static_cast<hipStream_t>(s), residual, input, output, gamma, hidden_size, epsilon, true));
 }
 
 trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {

@@ -1,0 +1,120 @@
+"""Host mirror of the element-wise decoder-layer kernels of trueno-gpu (kernels/elementwise.rs, kernels/layernorm.rs):
+ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel.
+
+Constructors, fields, `name()` strings and pointer parameter order are the reference's.  The reference compiles
+`hidden_size` and `epsilon` of the two norms into the PTX it emits; the pre-built kernels here take them as two
+more parameters after the pointers, which `kernel_args()` appends.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+from .driver import CudaModule, CudaStream, LaunchConfig, _check, _lib
+from .kernels import Kernel, _ptr
+
+
+class ResidualAddKernel(Kernel):
+    """output = input1 + input2 (elementwise.rs:33-101)."""
+
+    def __init__(self, n: int):
+        self.n = int(n)
+
+    def name(self) -> str:
+        return "residual_add"
+
+    def launch_config(self) -> LaunchConfig:
+        """block 256, grid ceil(n / 256) (elementwise.rs:27-30)."""
+        return LaunchConfig.linear(self.n, 256)
+
+    def kernel_args(self, input1, input2, output):
+        return [C.c_uint64(_ptr(input1)), C.c_uint64(_ptr(input2)), C.c_uint64(_ptr(output)), C.c_uint32(self.n)]
+
+    def launch(self, stream: CudaStream, input1, input2, output) -> None:
+        _check(_lib().trn_residual_add(stream.raw() if stream is not None else None, _ptr(input1), _ptr(input2),
+                                       _ptr(output), self.n), "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, input1, input2, output) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(input1, input2, output))
+
+
+class FusedSwigluKernel(Kernel):
+    """output = silu(gate) * up (elementwise.rs:521-592)."""
+
+    def __init__(self, n: int):
+        self.n = int(n)
+
+    def name(self) -> str:
+        return "fused_swiglu"
+
+    def launch_config(self) -> LaunchConfig:
+        return LaunchConfig.linear(self.n, 256)
+
+    def kernel_args(self, gate, up, output):
+        return [C.c_uint64(_ptr(gate)), C.c_uint64(_ptr(up)), C.c_uint64(_ptr(output)), C.c_uint32(self.n)]
+
+    def launch(self, stream: CudaStream, gate, up, output) -> None:
+        _check(_lib().trn_fused_swiglu(stream.raw() if stream is not None else None, _ptr(gate), _ptr(up), _ptr(output),
+                                       self.n), "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, gate, up, output) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(gate, up, output))
+
+
+class RmsNormKernel(Kernel):
+    """output = input / sqrt(mean(input^2) + epsilon) * gamma, one row (layernorm.rs:388-516)."""
+
+    def __init__(self, hidden_size: int):
+        self.hidden_size = int(hidden_size)
+        self.epsilon = 1e-5                     # layernorm.rs:400-405
+
+    def with_epsilon(self, epsilon: float) -> "RmsNormKernel":
+        self.epsilon = float(epsilon)
+        return self
+
+    def name(self) -> str:
+        return "rmsnorm"
+
+    def launch_config(self) -> LaunchConfig:
+        """one block of one warp (layernorm.rs:421-423)."""
+        return LaunchConfig((1, 1, 1), (32, 1, 1), 0)
+
+    def kernel_args(self, input, output, gamma):
+        return [C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma)), C.c_uint32(self.hidden_size),
+                C.c_float(self.epsilon)]
+
+    def launch(self, stream: CudaStream, input, output, gamma) -> None:
+        _check(_lib().trn_rmsnorm(stream.raw() if stream is not None else None, _ptr(input), _ptr(output), _ptr(gamma),
+                                  self.hidden_size, self.epsilon), "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, input, output, gamma) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(input, output, gamma))
+
+
+class FusedResidualRmsNormKernel(Kernel):
+    """output = rmsnorm(residual + input, gamma, epsilon), one row (elementwise.rs:109-248)."""
+
+    def __init__(self, hidden_size: int):
+        self.hidden_size = int(hidden_size)
+        self.epsilon = 1e-5                     # elementwise.rs:119-123
+
+    def with_epsilon(self, epsilon: float) -> "FusedResidualRmsNormKernel":
+        self.epsilon = float(epsilon)
+        return self
+
+    def name(self) -> str:
+        return "fused_residual_rmsnorm"
+
+    def launch_config(self) -> LaunchConfig:
+        return LaunchConfig((1, 1, 1), (32, 1, 1), 0)
+
+    def kernel_args(self, residual, input, output, gamma):
+        return [C.c_uint64(_ptr(residual)), C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma)),
+                C.c_uint32(self.hidden_size), C.c_float(self.epsilon)]
+
+    def launch(self, stream: CudaStream, residual, input, output, gamma) -> None:
+        _check(_lib().trn_fused_residual_rmsnorm(stream.raw() if stream is not None else None, _ptr(residual), _ptr(input),
+                                                 _ptr(output), _ptr(gamma), self.hidden_size, self.epsilon),
+               "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, residual, input, output, gamma) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(residual, input, output, gamma))
