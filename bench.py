@@ -123,8 +123,27 @@ def main() -> int:
     for kv in filter(None, os.environ.get("TRN_BENCH_TUNE", "").split(",")):      # working aid: library tuning keys
         key, val = kv.split("=")
         assert L.trn_set_tuning(key.encode(), int(val)) == 0, kv
+    def build_layer_pass():
+        """the decoder's serial data flow with the element-wise steps of a layer folded into the entries: q,k,v <-
+        rmsnorm(h)*g1; h1 = h + o(q); gate,up <- rmsnorm(h1)*g2; h = h1 + down(silu(gate)*up); head <- rmsnorm(h)*g"""
+        b = t.GemvBatch()
+        res = [t.GpuBuffer.from_host(ctx, kq.gen_x(777, 4096)), t.GpuBuffer(ctx, 4096, np.float32)]   # h, h1
+        gammas = [t.GpuBuffer.from_host(ctx, np.abs(kq.gen_x(780 + i, 4096)) + np.float32(0.5)) for i in range(2)]
+        w_of = lambda layer, name: weights[layer][name]
+        for layer in range(layers):
+            for name in ("q", "k", "v"):
+                b.add("q4k", 4096, 4096, act[name], w_of(layer, name), res[0], NORM, gamma=gammas[0], norm_eps=1e-5)
+            b.add("q4k", 4096, 4096, res[1], w_of(layer, "o"), act["q"], 0, residual=res[0])
+            for name in ("gate", "up"):
+                b.add("q4k", 4096, 11008, act[name], w_of(layer, name), res[1], NORM, gamma=gammas[1], norm_eps=1e-5)
+            b.add("q6k", 11008, 4096, res[0], w_of(layer, "down"), act["gate"], 0, x2=act["up"], residual=res[1])
+        b.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, res[0], NORM, gamma=gammas[0], norm_eps=1e-5)
+        b.keep = (res, gammas)
+        return b
+
     batch, total_bytes, weight_bytes = build_pass(False)
     strict_batch, _, _ = build_pass(True)
+    layer_batch = build_layer_pass()
 
     def ev():
         e = C.c_void_p()
@@ -207,6 +226,7 @@ def main() -> int:
 
     # ---- the same GEMVs wired as the strictly serial chain of a decoder ------------------------------------
     strict_ms, _ = run_passes(max(3, args.steps // 2), 2, strict_batch)
+    layer_ms, _ = run_passes(max(3, args.steps // 2), 2, layer_batch)
 
     # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
     other_modes = {}
@@ -352,7 +372,8 @@ def main() -> int:
                   "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
                   "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
-                  "weight_bytes": weight_bytes, "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us,
+                  "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": round(layer_ms * 1e3, 1),
+                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }

@@ -140,15 +140,29 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * process ends); a list identical to the previous one on that stream is not uploaded again.  If a device-side
  * wait ever runs out of its (seconds-long) spin budget the kernel exits and the next call on that stream returns
  * hipErrorLaunchFailure (719).  All three forms give bit-identical results. */
-#define TRN_GEMV_NORM_INPUT 1u /* the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x */
+/* An entry may fold the element-wise steps of a decoder layer in (zero pointers: absent):
+ *   x'  = x                          or silu(x) * x2            (TRN_GEMV_SWIGLU_INPUT; x = gate, x2 = up: fused_swiglu)
+ *   x'' = x' * gamma                 (gamma: k f32, the weights of rmsnorm)
+ *   y   = s * (W . x'') + residual   (residual: n f32; may be y itself),
+ *         s = 1, or 1 / sqrt(mean(x'^2) + norm_eps) with TRN_GEMV_NORM_INPUT (norm_eps 0 = 1e-6)
+ * so that rmsnorm -> projection, fused_residual_rmsnorm's second half, swiglu -> down projection and the residual
+ * add after o / down need no launches of their own.  gamma, x2 and residual count as read by the dependency
+ * analysis.  Such entries need x, x2 and gamma 16-byte aligned. */
+#define TRN_GEMV_NORM_INPUT 1u   /* the entry reads x' / sqrt(mean(x'^2) + eps) instead of x' */
+#define TRN_GEMV_SWIGLU_INPUT 8u /* the entry reads silu(x) * x2 instead of x */
 typedef struct trn_gemv_desc {
   uint32_t fmt;
   uint32_t k;
   uint32_t n;
-  uint32_t flags;      /* 0 or TRN_GEMV_NORM_INPUT */
+  uint32_t flags;      /* 0 or TRN_GEMV_NORM_INPUT | TRN_GEMV_SWIGLU_INPUT */
   trn_dptr y;
   trn_dptr w;
   trn_dptr x;
+  trn_dptr gamma;
+  trn_dptr x2;
+  trn_dptr residual;
+  float norm_eps;
+  uint32_t reserved;   /* 0 */
 } trn_gemv_desc;
 TRN_API trn_status trn_kquant_gemv_batch(trn_stream stream, const trn_gemv_desc* descs, uint32_t count);
 

@@ -205,7 +205,7 @@ def test_chain_rejects_bad_entries(gpu):
     assert L.trn_kquant_gemv_batch(stream.raw(), d, 2) == 1
     d[1] = _ffi.GemvDesc(4, 100, 4, 0, 16, 16, 16)
     assert L.trn_kquant_gemv_batch(stream.raw(), d, 2) == 1
-    d[1] = _ffi.GemvDesc(4, 256, 4, 8, 16, 16, 16)
+    d[1] = _ffi.GemvDesc(4, 256, 4, 16, 16, 16, 16)
     assert L.trn_kquant_gemv_batch(stream.raw(), d, 2) == 1
     assert L.trn_kquant_gemv_batch(stream.raw(), None, 0) == 0
 

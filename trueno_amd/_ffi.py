@@ -75,7 +75,9 @@ _RESTYPE = {"trn_error_name": C.c_char_p, "trn_error_string": C.c_char_p}
 class GemvDesc(C.Structure):
     """trn_gemv_desc"""
     _fields_ = [("fmt", C.c_uint32), ("k", C.c_uint32), ("n", C.c_uint32), ("flags", C.c_uint32),
-                ("y", C.c_uint64), ("w", C.c_uint64), ("x", C.c_uint64)]
+                ("y", C.c_uint64), ("w", C.c_uint64), ("x", C.c_uint64),
+                ("gamma", C.c_uint64), ("x2", C.c_uint64), ("residual", C.c_uint64),
+                ("norm_eps", C.c_float), ("reserved", C.c_uint32)]
 
 
 class LibraryMissing(OSError):

@@ -34,14 +34,31 @@
 #define CHAIN_STAMP(slot) do { } while (0)
 #endif
 
+// One GEMV of a list with the element-wise steps of a decoder layer folded in:
+//   x'  = x                         or  silu(x) * x2                         (CHAIN_SWIGLU_INPUT; fused_swiglu)
+//   x'' = x' * gamma                (gamma != null)
+//   y   = s * (W . x'') + residual  (residual != null),  s = 1 or 1/sqrt(mean(x'^2) + eps)   (CHAIN_NORM_INPUT)
+// i.e. rmsnorm(x') * gamma feeds the product (rmsnorm / fused_residual_rmsnorm in front of a projection) and a
+// residual add follows it.
 struct ChainEntry {
   u32 fmt, k, n, flags;
   const uint8_t* w;
   const float* x;
   float* y;
+  const float* gamma;
+  const float* x2;
+  const float* residual;
+  float eps;          // of the normalisation; 0 = kChainNormEps
+  u32 pad;
 };
-enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u };
+enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u, CHAIN_SWIGLU_INPUT = 8u };
 constexpr float kChainNormEps = 1e-6f;
+
+// silu(g) * u with the reference's instruction sequence (trueno-gpu/src/kernels/elementwise.rs:565-582)
+__device__ __forceinline__ float swiglu1(float g, float u) {
+  const float denom = __fadd_rn(1.0f, __builtin_amdgcn_exp2f(__fmul_rn(__fsub_rn(0.0f, g), 1.442695f)));
+  return __fmul_rn(__fmul_rn(g, __fdiv_rn(1.0f, denom)), u);
+}
 
 // Sum of squares of the activation vector in ONE fixed order, whatever the launch shape: the vector is cut in
 // groups of 64 16-byte units (256 values); the sum of a group is the fixed wave butterfly over its units (unit
@@ -153,6 +170,19 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
     } else {
       v = x4[u];
     }
+    if (e.flags & CHAIN_SWIGLU_INPUT) {
+      f32x4 g2;
+      if constexpr (COHERENT) {
+        const u32* xw = reinterpret_cast<const u32*>(e.x2) + 4u * u;
+        g2.x = __uint_as_float(__hip_atomic_load(xw + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        g2.y = __uint_as_float(__hip_atomic_load(xw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        g2.z = __uint_as_float(__hip_atomic_load(xw + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        g2.w = __uint_as_float(__hip_atomic_load(xw + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      } else {
+        g2 = reinterpret_cast<const f32x4*>(e.x2)[u];
+      }
+      v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
+    }
     return v;
   };
   constexpr u32 kXPre = 4;                              // groups per wave requested ahead of the weights
@@ -177,12 +207,16 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   float* part = reinterpret_cast<float*>(lds4 + units);
   float* group_ss = part + sw_count * rows_per_block;   // one sum of squares per group of 64 units
   const bool norm = (e.flags & CHAIN_NORM_INPUT) != 0u;
-  auto stage = [&](u32 g, const f32x4 v) {
-    lds4[Q::swz(64u * g + lane)] = v;
+  auto stage = [&](u32 g, f32x4 v) {
     if (norm) {
       const float sg = wave_sum(unit_sumsq(v));
       if (lane == 0) group_ss[g] = sg;
     }
+    if (e.gamma) {                      // weights of the normalisation, never written inside a launch
+      const f32x4 gm = reinterpret_cast<const f32x4*>(e.gamma)[64u * g + lane];
+      v = f32x4{__fmul_rn(v.x, gm.x), __fmul_rn(v.y, gm.y), __fmul_rn(v.z, gm.z), __fmul_rn(v.w, gm.w)};
+    }
+    lds4[Q::swz(64u * g + lane)] = v;
   };
   if (x_first) {
 #pragma unroll
@@ -201,7 +235,7 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   if (norm) {
     float total = group_ss[0];
     for (u32 g = 1; g < xgroups; ++g) total += group_ss[g];
-    scale = 1.0f / sqrtf(total / static_cast<float>(k_dim) + kChainNormEps);
+    scale = 1.0f / sqrtf(total / static_cast<float>(k_dim) + (e.eps != 0.0f ? e.eps : kChainNormEps));
   }
   CHAIN_STAMP(4);
 
@@ -242,11 +276,16 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
     if (row < n_dim) {
       float s = part[t];
       for (u32 i = 1; i < sw_count; ++i) s += part[i * rows_per_block + t];
-      if constexpr (COHERENT)
-        __hip_atomic_store(reinterpret_cast<u32*>(e.y) + row, __float_as_uint(s * scale), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-      else
-        e.y[row] = s * scale;
+      float r = s * scale;
+      if constexpr (COHERENT) {
+        if (e.residual)
+          r = __fadd_rn(r, __uint_as_float(__hip_atomic_load(reinterpret_cast<const u32*>(e.residual) + row, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT)));
+        __hip_atomic_store(reinterpret_cast<u32*>(e.y) + row, __float_as_uint(r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        if (e.residual) r = __fadd_rn(r, e.residual[row]);
+        e.y[row] = r;
+      }
     }
   }
   CHAIN_STAMP(3);

@@ -359,9 +359,28 @@ hipError_t launch_dequant(Fmt f, hipStream_t stream, uint64_t out, uint64_t w, u
 // ---- the persistent executor behind trn_kquant_gemv_batch ---------------------------------------
 struct ChainEntryHost {  // ChainEntry of kquant_chain.hip.h
   uint32_t fmt, k, n, flags;
-  uint64_t w, x, y;
+  uint64_t w, x, y, gamma, x2, residual;
+  float eps;
+  uint32_t pad;
 };
-static_assert(sizeof(ChainEntryHost) == 40, "ChainEntry layout");
+static_assert(sizeof(ChainEntryHost) == 72, "ChainEntry layout");
+ChainEntryHost entry_of(const trn_gemv_desc& d, uint32_t extra_flags = 0u) {
+  return {d.fmt, d.k, d.n, d.flags | extra_flags, d.w, d.x, d.y, d.gamma, d.x2, d.residual, d.norm_eps, 0u};
+}
+// an entry that folds element-wise steps in (only the quarter-block engine knows how)
+bool desc_extended(const trn_gemv_desc& d) { return d.gamma || d.x2 || d.residual || (d.flags & TRN_GEMV_SWIGLU_INPUT); }
+// does g read or write what p writes, or write what p reads?
+bool desc_conflict(const trn_gemv_desc& g, const trn_gemv_desc& p) {
+  const uint64_t reads_g[4][2] = {{g.x, 4ull * g.k}, {g.x2, g.x2 ? 4ull * g.k : 0}, {g.gamma, g.gamma ? 4ull * g.k : 0},
+                                  {g.residual, g.residual ? 4ull * g.n : 0}};
+  const uint64_t reads_p[4][2] = {{p.x, 4ull * p.k}, {p.x2, p.x2 ? 4ull * p.k : 0}, {p.gamma, p.gamma ? 4ull * p.k : 0},
+                                  {p.residual, p.residual ? 4ull * p.n : 0}};
+  auto overlap = [](uint64_t a, uint64_t alen, uint64_t b, uint64_t blen) { return alen && blen && a < b + blen && b < a + alen; };
+  if (overlap(g.y, 4ull * g.n, p.y, 4ull * p.n)) return true;
+  for (int i = 0; i < 4; ++i)
+    if (overlap(reads_g[i][0], reads_g[i][1], p.y, 4ull * p.n) || overlap(g.y, 4ull * g.n, reads_p[i][0], reads_p[i][1])) return true;
+  return false;
+}
 
 struct ChainWorkspace {
   void* d_entries = nullptr;
@@ -383,12 +402,8 @@ std::map<std::pair<int, hipStream_t>, ChainWorkspace> g_chain_ws;
 // (chain_barrier_stride of kquant_chain.hip.h)
 uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u + (num_workgroups + 31u) / 32u); }
 
-bool ranges_overlap(uint64_t a, uint64_t alen, uint64_t b, uint64_t blen) { return a < b + blen && b < a + alen; }
 
-bool desc_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) {
-  return ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
-         ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
-}
+bool desc_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
 // batch_mode 1: the list as phases of independent entries in ONE resident launch (kq_gemv_phases): one workgroup
 // of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
@@ -412,7 +427,7 @@ hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t strea
   const uint32_t phases = uint32_t(ph.size());
   std::vector<uint32_t> assign(size_t(phases) * G * 4u, 0u);   // entry, block_id, num_blocks, fmt
   std::vector<ChainEntryHost> entries(count);
-  for (uint32_t i = 0; i < count; ++i) entries[i] = {descs[i].fmt, descs[i].k, descs[i].n, descs[i].flags, descs[i].w, descs[i].x, descs[i].y};
+  for (uint32_t i = 0; i < count; ++i) entries[i] = entry_of(descs[i]);
   uint32_t lds = 0;
   for (uint32_t p = 0; p < phases; ++p) {
     const uint32_t a = ph[p].first, b = ph[p].second, m = b - a;
@@ -530,14 +545,13 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
     bool dep = false;
     for (size_t j = group_begin; j < i && !dep; ++j) {
       const trn_gemv_desc& p = descs[j];
-      dep = ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
-            ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
+      dep = desc_conflict(g, p);
     }
     if (dep) {
       ++barriers;
       group_begin = i;
     }
-    entries[i] = {g.fmt, g.k, g.n, g.flags | (dep ? kFlagBarrierBefore : 0u), g.w, g.x, g.y};
+    entries[i] = entry_of(g, dep ? kFlagBarrierBefore : 0u);
   }
   int dev = 0;
   (void)hipGetDevice(&dev);
@@ -560,6 +574,7 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
 
   // ---- streaming form: one workgroup per CU, a producer wave feeding an LDS ring -------------------
   bool use_stream = g_tune_batch_mode == 2;
+  for (uint32_t i = 0; i < count; ++i) use_stream = use_stream && !desc_extended(descs[i]);   // the streaming kernel has no folded steps
   uint32_t consumers = g_tune_stream_consumers > 0 ? uint32_t(g_tune_stream_consumers) : 7u;
   consumers = std::max(1u, std::min(consumers, 7u));
   const uint32_t sgrid = uint32_t(d->cu_count);
@@ -944,12 +959,9 @@ struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip
   uint32_t first[5];
   uint32_t count;
 };
-static_assert(sizeof(GemvGroupHost) == 4 * 40 + 5 * 4 + 4, "GemvGroup layout");
+static_assert(sizeof(GemvGroupHost) == 4 * 72 + 5 * 4 + 4, "GemvGroup layout");
 
-bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) {
-  return ranges_overlap(g.x, 4ull * g.k, p.y, 4ull * p.n) || ranges_overlap(g.y, 4ull * g.n, p.y, 4ull * p.n) ||
-         ranges_overlap(g.y, 4ull * g.n, p.x, 4ull * p.k);
-}
+bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
 // Entries first .. first+len-1 of a list (len in 2..4, mutually independent, all meeting the fast kernels'
 // preconditions) as ONE launch.  The workgroups are as large as the largest entry needs (k > 4096 wants one
@@ -984,7 +996,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     rows = std::min<uint64_t>(rows, max_rows);
     const uint32_t grid = uint32_t((uint64_t(e.n) + rows - 1) / rows);
     lds = std::max<uint32_t>(lds, uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch));
-    g.e[i] = {e.fmt, e.k, e.n, e.flags, e.w, e.x, e.y};
+    g.e[i] = entry_of(e);
     g.first[i + 1] = g.first[i] + grid;
   }
   g.count = len;
@@ -1019,7 +1031,9 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   if (count == 0) return TRN_SUCCESS;
   if (!descs) return TRN_ERROR_INVALID_VALUE;
   for (uint32_t i = 0; i < count; ++i)  // validate the whole list before anything is launched
-    if (descs[i].fmt < 4 || descs[i].fmt > 6 || (descs[i].flags & ~TRN_GEMV_NORM_INPUT) != 0 || descs[i].k % 256u != 0)
+    if (descs[i].fmt < 4 || descs[i].fmt > 6 || (descs[i].flags & ~(TRN_GEMV_NORM_INPUT | TRN_GEMV_SWIGLU_INPUT)) != 0 ||
+        descs[i].k % 256u != 0 || ((descs[i].flags & TRN_GEMV_SWIGLU_INPUT) != 0) != (descs[i].x2 != 0) ||
+        !aligned(descs[i].gamma, 16) || !aligned(descs[i].x2, 16) || !aligned(descs[i].residual, 4) || !(descs[i].norm_eps >= 0.0f))
       return TRN_ERROR_INVALID_VALUE;
   hipStream_t stream = static_cast<hipStream_t>(s);
   bool handled = false;
@@ -1043,8 +1057,11 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
         ++len;
       }
     }
-    if (len >= 2) {
+    if (len >= 2 || (desc_extended(descs[i]) && groupable(descs[i]))) {
       e = launch_gemv_group(dk, stream, descs + i, len);
+    } else if (desc_extended(descs[i])) {
+      // folded element-wise steps need the fast engine (x, x2, gamma 16-byte aligned; the vector and a row block in LDS)
+      return TRN_ERROR_INVALID_VALUE;
     } else {
       const trn_gemv_desc& d = descs[i];
       e = launch_gemm_like(Fmt(d.fmt - 4), stream, d.x, d.w, d.y, 1, d.n, d.k, true, d.flags);

@@ -219,10 +219,18 @@ class GemvBatch:
         self._entries = []
         self._array = None
 
-    NORM_INPUT = 1  # the entry reads x / sqrt(mean(x^2) + 1e-6) instead of x
+    NORM_INPUT = 1    # the entry reads x / sqrt(mean(x^2) + eps) instead of x
+    SWIGLU_INPUT = 8  # the entry reads silu(x) * x2 instead of x (x = gate, x2 = up)
 
-    def add(self, fmt: str, k: int, n: int, y, w, x, flags: int = 0) -> "GemvBatch":
-        self._entries.append(_ffi.GemvDesc(self._FMT[fmt], int(k), int(n), int(flags), _ptr(y), _ptr(w), _ptr(x)))
+    def add(self, fmt: str, k: int, n: int, y, w, x, flags: int = 0, gamma=None, x2=None, residual=None,
+            norm_eps: float = 0.0) -> "GemvBatch":
+        """y = s * W (x' * gamma) + residual with x' = x or silu(x) * x2 and s = 1 or the RMS normalisation of x':
+        the element-wise steps of a decoder layer (rmsnorm, fused_swiglu, residual_add) folded into the GEMV."""
+        if x2 is not None:
+            flags |= self.SWIGLU_INPUT
+        self._entries.append(_ffi.GemvDesc(self._FMT[fmt], int(k), int(n), int(flags), _ptr(y), _ptr(w), _ptr(x),
+                                           0 if gamma is None else _ptr(gamma), 0 if x2 is None else _ptr(x2),
+                                           0 if residual is None else _ptr(residual), float(norm_eps), 0))
         self._array = None
         return self
 
