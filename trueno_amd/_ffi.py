@@ -5,7 +5,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtrueno_hip.so")
+LIB_PATH = os.environ.get("TRN_HIP_LIBRARY") or os.path.join(_HERE, "libtrueno_hip.so")   # another build, for comparisons
 
 _lib = None
 

@@ -229,6 +229,11 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   // Workgroup barrier over the LDS writes only.  __syncthreads() would also drain the weight loads that are in
   // flight (the compiler waits for every outstanding memory operation before s_barrier), which is the one thing
   // the ordering above is there to avoid.
+  // Batches of rows after a wave's first are handed out as waves become free (one counter per slab index, so
+  // that the waves sharing a row's slabs each see every batch once): the memory system does not serve the waves
+  // evenly, and the workgroup is only done when its slowest wave is.
+  __shared__ u32 s_next[16];
+  if (tid < 16u) s_next[tid] = groups;
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   CHAIN_STAMP(2);
   float scale = 1.0f;
@@ -256,8 +261,11 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
         xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
         sx[Q::sum_index(4 * q)] += (v.x + v.y) + (v.z + v.w);
       }
-      for (u32 b = grp; b < batches; b += groups) {
+      const bool handed_out = slabs <= waves && waves >= 8u;   // every wave owns one slab; small workgroups gain nothing
+      for (u32 b = grp; b < batches;) {
         if (slab != sw || b != grp) issue(slab, b);
+        u32 nb = 0u;                                // the batch after this one, asked for while this one is computed
+        if (handed_out && lane == 0) nb = __hip_atomic_fetch_add(&s_next[sw], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
@@ -265,6 +273,11 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
             const u32 idx = sw * rows_per_block + b * U + u;
             part[idx] = (slab == sw) ? p : part[idx] + p;
           }
+        }
+        if (handed_out) {
+          b = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(nb)));
+        } else {
+          b += groups;
         }
       }
     }
