@@ -319,6 +319,31 @@ def main() -> int:
             stream.synchronize()
             glue_us[label] = round(elapsed_ms(e0, e1) * 1e3 / 64, 2)
 
+    # ---- the f32 GEMV of gemv.rs (A is K x N row-major), one launch, cold --------------------------------------
+    f32_gemv = {}
+    if not args.no_configs:
+        rng = np.random.default_rng(55)
+        for k, n, copies in ((4096, 4096, 8), (4096, 11008, 4)):
+            host = rng.standard_normal(k * n, dtype=np.float32)
+            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            xb, yb = xs[0][0], y[n if n in y else 11008]
+            def launch(r):
+                return L.trn_gemv_f32(stream.raw(), yb.as_ptr(), bufs[r % copies].as_ptr(), xb.as_ptr(), k, n)
+            for r in range(copies):
+                launch(r)
+            stream.synchronize()
+            L.trn_event_record(e0, stream.raw())
+            for r in range(2 * copies):
+                launch(r)
+            L.trn_event_record(e1, stream.raw())
+            stream.synchronize()
+            us = elapsed_ms(e0, e1) * 1e3 / (2 * copies)
+            nbytes = 4 * k * n + 4 * k + 4 * n
+            f32_gemv[f"k{k}_n{n}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                      "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            for b in bufs:
+                b.free()
+
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
     cpu_config1 = None
@@ -373,7 +398,7 @@ def main() -> int:
                   "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
                   "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": round(layer_ms * 1e3, 1),
-                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us,
+                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "f32_gemv_single_launch_cold": f32_gemv,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }

@@ -182,6 +182,12 @@ TRN_API trn_status trn_event_destroy(trn_event event);
 TRN_API trn_status trn_event_record(trn_event event, trn_stream stream);
 TRN_API trn_status trn_event_synchronize(trn_event event);
 TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop);
+/* f32 GEMV: y[n] = sum_k a[k*n_dim + n] * x[k]; a is K x N row-major, i.e. transposed relative to the quantized
+ * matrices.  trueno-gpu/src/kernels/gemv.rs: GemvKernel "gemv_warp_reduce" :21-166 and CoalescedGemvKernel
+ * "gemv_coalesced" :188-398, both (y_ptr, a_ptr, x_ptr, k_dim, n_dim); the built-in module has both names.  Keeps a
+ * small per-stream workspace (allocated on first use). */
+TRN_API trn_status trn_gemv_f32(trn_stream stream, trn_dptr y, trn_dptr a, trn_dptr x, uint32_t k, uint32_t n);
+
 /* ---- element-wise steps between the GEMVs of a decoder layer (f32 vectors) ---------------------------------
  * The same kernels are in the built-in module under the reference's names "residual_add", "fused_swiglu",
  * "rmsnorm", "fused_residual_rmsnorm".  The first two keep the reference's parameter lists; the reference

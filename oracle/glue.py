@@ -8,6 +8,9 @@ Reference lines followed (under trueno-gpu/src/kernels/):
   fused_swiglu            elementwise.rs:521-592   sub, mul by 1.442695f, ex2.approx, add, div.rn, mul, mul
   rmsnorm                 layernorm.rs:388-516     32 lanes, fma per element, shfl.down tree, div.rn, add, rsqrt.approx, mul, mul
   fused_residual_rmsnorm  elementwise.rs:109-248   the same on x = residual + input
+  gemv_warp_reduce        gemv.rs:21-166           y[n] = sum_k A[k][n] x[k], A K x N row-major; lane t of 32 takes
+                                                   k = t, t+32, ... by fma, then the shfl.down tree
+  gemv_coalesced          gemv.rs:188-398          the same product, one thread per column, k in order by fma
 (div.f32 is printed as div.rn, ex2/rsqrt as .approx: trueno-gpu/src/ptx/builder.rs:1425-1431, 1523-1530.)
 
 Every f32 operation is rounded separately, as the reference's instructions are.  The two approximate
@@ -22,6 +25,8 @@ How each function is pinned (the reference holds no numeric test of these kernel
                           bit: the difference is covered and bounded in the tests).
   rmsnorm*              : closed forms (constant rows, one-hot rows), mean square of the output, scale invariance,
                           agreement with the fp64 formula; the lane order is an emulation used for error magnitudes.
+  gemv_f32_*            : an fp64 matrix product is the closed form; brute force on tiny shapes; the two f32 orders
+                          are emulations used for error magnitudes only.
 Against a running reference these stay "parity unpinned": it cannot be run here (no Rust, no NVIDIA driver).
 """
 import numpy as np
@@ -91,3 +96,31 @@ def rmsnorm_fp64(x, gamma, eps=1e-5, residual=None):
     if residual is not None:
         x = (np.asarray(residual, F32) + np.asarray(x, F32)).astype(np.float64)     # the add is an f32 add in the reference
     return x / np.sqrt(np.mean(x * x) + np.float64(F32(eps))) * np.asarray(gamma, np.float64)
+
+
+def gemv_f32_fp64(a, x):
+    """y[n] = sum_k A[k][n] x[k] (gemv.rs:1-15): A is K x N row-major."""
+    return np.asarray(x, np.float64) @ np.asarray(a, np.float64)
+
+
+def gemv_f32_coalesced_order(a, x):
+    """gemv.rs:292-378: per column, sum = fma(x[k], A[k][n], sum) for k = 0, 1, 2, ..."""
+    a, x = np.asarray(a, F32), np.asarray(x, F32)
+    acc = np.zeros(a.shape[1], F32)
+    for k in range(a.shape[0]):
+        acc = (np.float64(x[k]) * a[k].astype(np.float64) + acc.astype(np.float64)).astype(F32)
+    return acc
+
+
+def gemv_f32_warp_reduce_order(a, x):
+    """gemv.rs:84-132: lane t accumulates k = t, t+32, ... by fma; then shfl.down 16, 8, 4, 2, 1."""
+    a, x = np.asarray(a, F32), np.asarray(x, F32)
+    lanes = np.zeros((32, a.shape[1]), F32)
+    for k in range(a.shape[0]):
+        t = k % 32
+        lanes[t] = (np.float64(x[k]) * a[k].astype(np.float64) + lanes[t].astype(np.float64)).astype(F32)
+    for d in (16, 8, 4, 2, 1):
+        nxt = lanes.copy()
+        nxt[:32 - d] = (lanes[:32 - d] + lanes[d:]).astype(F32)
+        lanes = nxt
+    return lanes[0]

@@ -7,8 +7,8 @@ over the C ABI of libtrueno_hip.so:
                         (trueno-gpu/src/driver/{context,module,stream,memory,types}.rs, src/error.rs)
     trueno_amd.kernels  Kernel, Q4KGemvKernel, Q5KGemvKernel, Q6KGemvKernel, QuantizeKernel,
                         Q5KKernel, Q6KKernel, Q4KFormat   (trueno-gpu/src/kernels/quantize.rs)
-    trueno_amd.glue     ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel
-                        (trueno-gpu/src/kernels/elementwise.rs, layernorm.rs)
+    trueno_amd.glue     ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel, GemvKernel,
+                        CoalescedGemvKernel   (trueno-gpu/src/kernels/elementwise.rs, layernorm.rs, gemv.rs)
 
 There is no CPU path: without libtrueno_hip.so or without a GPU every device call raises GpuError.
 """
@@ -17,4 +17,5 @@ from .driver import (CudaContext, CudaModule, CudaStream, GpuBuffer, GpuError, L
                      cuda_available, device_count)
 from .kernels import (GemvBatch, Kernel, Q4KFormat, Q4KGemvKernel, Q5KGemvKernel, Q5KKernel, Q6KGemvKernel,  # noqa: F401
                       Q6KKernel, QuantizeKernel)
-from .glue import FusedResidualRmsNormKernel, FusedSwigluKernel, ResidualAddKernel, RmsNormKernel  # noqa: F401
+from .glue import (CoalescedGemvKernel, FusedResidualRmsNormKernel, FusedSwigluKernel, GemvKernel,  # noqa: F401
+                   ResidualAddKernel, RmsNormKernel)

@@ -12,6 +12,7 @@
 #include "kquant_stream.hip.h"
 #include "kquant_gemm_f16.hip.h"
 #include "decode_glue.hip.h"
+#include "gemv_f32.hip.h"
 
 // The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
 // activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
@@ -135,6 +136,21 @@ rmsnorm(const float* input, float* output, const float* gamma, u32 hidden_size, 
 extern "C" __global__ void __launch_bounds__(1024)
 fused_residual_rmsnorm(const float* residual, const float* input, float* output, const float* gamma, u32 hidden_size, float epsilon) {
   glue::rmsnorm_body<true>(residual, input, output, gamma, hidden_size, epsilon);
+}
+
+// f32 GEMV under the reference's two kernel names and parameter list (gemv.rs:53-57, 222-226): one engine
+// (gemv_f32.hip.h), the two names differ only in the reference's summation order.  gemv_f32_fast takes the
+// launcher's extra arguments; the named kernels are the any-shape form.
+extern "C" __global__ void __launch_bounds__(512)
+gemv_f32_fast(float* y, const float* a, const float* x, float* partial, u32* counters, u32 k_dim, u32 n_dim, u32 rows_per_part,
+              u32 parts) {
+  gemv_f32::fast_body(y, a, x, partial, counters, k_dim, n_dim, rows_per_part, parts);
+}
+extern "C" __global__ void __launch_bounds__(256) gemv_warp_reduce(float* y, const float* a, const float* x, u32 k_dim, u32 n_dim) {
+  gemv_f32::generic_body(y, a, x, k_dim, n_dim);
+}
+extern "C" __global__ void __launch_bounds__(256) gemv_coalesced(float* y, const float* a, const float* x, u32 k_dim, u32 n_dim) {
+  gemv_f32::generic_body(y, a, x, k_dim, n_dim);
 }
 
 extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32 v) {

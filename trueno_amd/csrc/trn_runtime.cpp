@@ -44,7 +44,7 @@ const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 
 // kinds of functions the launch-by-name path recognises
 enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3, KIND_RESIDUAL_ADD = 4, KIND_SWIGLU = 5,
-            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7 };
+            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8 };
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
@@ -67,6 +67,7 @@ struct DeviceKernels {
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
+  hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr;
   hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
@@ -122,6 +123,8 @@ hipError_t device_kernels(DeviceKernels** out) {
       }
     }
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
+        (e = get_fn(m, &t.gemv_f32_fast, "gemv_f32_fast")) != hipSuccess ||
+        (e = get_fn(m, &t.gemv_f32_generic, "gemv_coalesced")) != hipSuccess ||
         (e = get_fn(m, &t.residual_add, "residual_add")) != hipSuccess ||
         (e = get_fn(m, &t.swiglu, "fused_swiglu")) != hipSuccess ||
         (e = get_fn(m, &t.rmsnorm, "rmsnorm")) != hipSuccess ||
@@ -227,6 +230,56 @@ hipError_t launch_rmsnorm(hipStream_t stream, uint64_t residual, uint64_t in, ui
   }
   void* args[] = {&in, &out, &gamma, &hidden, &eps};
   return hipModuleLaunchKernel(d->rmsnorm, 1, 1, 1, block, 1, 1, 0, stream, args, nullptr);
+}
+
+// f32 GEMV y = A^T-style product with A K x N row-major (gemv_f32.hip.h).  Partial results of the parts of K and
+// the arrival counters live in a per-(device, stream) buffer like the GEMM's.
+struct GemvF32Workspace {
+  void* buf = nullptr;
+  size_t cap = 0;
+};
+std::map<std::pair<int, hipStream_t>, GemvF32Workspace> g_gemv_f32_ws;
+
+hipError_t launch_gemv_f32(hipStream_t stream, uint64_t y, uint64_t a, uint64_t x, uint32_t k, uint32_t n) {
+  if (n == 0) return hipSuccess;
+  if (!y || (k != 0 && (!a || !x)) || !aligned(y, 4) || !aligned(a, 4) || !aligned(x, 4)) return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  if (k == 0 || n % 4u != 0 || !aligned(a, 16) || !aligned(y, 16)) {
+    void* args[] = {&y, &a, &x, &k, &n};
+    return hipModuleLaunchKernel(d->gemv_f32_generic, (n + 255u) / 256u, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
+  }
+  const uint32_t tiles = (n + 255u) / 256u;
+  // parts of K: about two workgroups of 8 waves per CU, at least 64 rows (8 per wave) each
+  uint32_t parts = std::max(1u, (2u * uint32_t(d->cu_count) + tiles / 2u) / tiles);
+  parts = std::max(1u, std::min(parts, (k + 63u) / 64u));
+  uint32_t rows_per_part = (k + parts - 1u) / parts;
+  rows_per_part = (rows_per_part + 7u) / 8u * 8u;
+  parts = (k + rows_per_part - 1u) / rows_per_part;
+  const size_t cnt_cap = 64u * 1024u, need = cnt_cap + (parts > 1u ? size_t(parts) * n * 4u : 0u);
+  if (size_t(tiles) * 4u > cnt_cap) return hipErrorInvalidValue;
+  int dev = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+  GemvF32Workspace* ws;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    ws = &g_gemv_f32_ws[std::make_pair(dev, stream)];
+  }
+  if (ws->cap < need) {
+    if (ws->buf) {
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;
+      (void)hipFree(ws->buf);
+      ws->buf = nullptr;
+      ws->cap = 0;
+    }
+    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
+    ws->cap = need;
+    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;   // the kernel leaves the counters at zero
+  }
+  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  void* args[] = {&y, &a, &x, &part, &cnt, &k, &n, &rows_per_part, &parts};
+  return hipModuleLaunchKernel(d->gemv_f32_fast, tiles * parts, 1, 1, 512, 1, 1, 0, stream, args, nullptr);
 }
 
 // Partial results and arrival counters of the matrix-core GEMM: one buffer per (device, stream), grown on
@@ -795,6 +848,7 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
       if (n == std::string(kFmtName[i]) + "_gemm_ggml") { h->kind = KIND_GEMM; h->fmt = i; }
     }
     if (n == "q4k_gemm_fused") h->kind = KIND_GEMM_SIMPLIFIED;
+    if (n == "gemv_warp_reduce" || n == "gemv_coalesced") h->kind = KIND_GEMV_F32;
     if (n == "residual_add") h->kind = KIND_RESIDUAL_ADD;
     if (n == "fused_swiglu") h->kind = KIND_SWIGLU;
     if (n == "rmsnorm") h->kind = KIND_RMSNORM;
@@ -905,6 +959,19 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     if (func->kind == KIND_GEMM_SIMPLIFIED) return st(launch_gemm_simplified(s, p0, p1, p2, m, n, k));
     return st(launch_gemm_like(Fmt(func->fmt), s, p0, p1, p2, m, n, k, false));
   }
+  if (func->kind == KIND_GEMV_F32) {                                           // (y, a, x, k_dim, n_dim)
+    if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
+    for (int i = 0; i < 5; ++i)
+      if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
+    uint64_t p0, p1, p2;
+    uint32_t k, n;
+    std::memcpy(&p0, kernel_params[0], 8);
+    std::memcpy(&p1, kernel_params[1], 8);
+    std::memcpy(&p2, kernel_params[2], 8);
+    std::memcpy(&k, kernel_params[3], 4);
+    std::memcpy(&n, kernel_params[4], 4);
+    return st(launch_gemv_f32(s, p0, p1, p2, k, n));
+  }
   if (func->kind == KIND_RESIDUAL_ADD || func->kind == KIND_SWIGLU) {          // (ptr, ptr, output_ptr, n)
     if (!kernel_params || !kernel_params[0] || !kernel_params[1] || !kernel_params[2] || !kernel_params[3]) return TRN_ERROR_INVALID_VALUE;
     uint64_t p0, p1, p2;
@@ -1013,6 +1080,9 @@ trn_status trn_q4k_simplified_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w
   return st(launch_dequant_simplified(static_cast<hipStream_t>(s), out, w, n_blocks));
 }
 
+trn_status trn_gemv_f32(trn_stream s, trn_dptr y, trn_dptr a, trn_dptr x, uint32_t k, uint32_t n) {
+  return st(launch_gemv_f32(static_cast<hipStream_t>(s), y, a, x, k, n));
+}
 trn_status trn_residual_add(trn_stream s, trn_dptr input1, trn_dptr input2, trn_dptr output, uint32_t n) {
   return st(launch_elementwise(KIND_RESIDUAL_ADD, static_cast<hipStream_t>(s), input1, input2, output, n));
 }

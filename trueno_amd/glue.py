@@ -1,5 +1,6 @@
 """Host mirror of the element-wise decoder-layer kernels of trueno-gpu (kernels/elementwise.rs, kernels/layernorm.rs):
-ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel.
+ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel - and of its f32 GEMV kernels
+(kernels/gemv.rs): GemvKernel, CoalescedGemvKernel.
 
 Constructors, fields, `name()` strings and pointer parameter order are the reference's.  The reference compiles
 `hidden_size` and `epsilon` of the two norms into the PTX it emits; the pre-built kernels here take them as two
@@ -118,3 +119,42 @@ class FusedResidualRmsNormKernel(Kernel):
 
     def launch_by_name(self, stream: CudaStream, module: CudaModule, residual, input, output, gamma) -> None:
         stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(residual, input, output, gamma))
+
+
+class _GemvF32(Kernel):
+    """y = A x-style product with A K x N row-major: y[n] = sum_k A[k][n] x[k] (gemv.rs)."""
+    _NAME = ""
+
+    def __init__(self, k: int, n: int):
+        self.k = int(k)
+        self.n = int(n)
+
+    def name(self) -> str:
+        return self._NAME
+
+    def kernel_args(self, y, a, x):
+        """(y_ptr, a_ptr, x_ptr, k_dim, n_dim) - gemv.rs:53-57, 222-226."""
+        return [C.c_uint64(_ptr(y)), C.c_uint64(_ptr(a)), C.c_uint64(_ptr(x)), C.c_uint32(self.k), C.c_uint32(self.n)]
+
+    def launch(self, stream: CudaStream, y, a, x) -> None:
+        _check(_lib().trn_gemv_f32(stream.raw() if stream is not None else None, _ptr(y), _ptr(a), _ptr(x), self.k, self.n),
+               "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, y, a, x) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(y, a, x))
+
+
+class GemvKernel(_GemvF32):
+    """gemv.rs:21-166: one warp per output element."""
+    _NAME = "gemv_warp_reduce"
+
+    def launch_config(self) -> LaunchConfig:
+        return LaunchConfig((self.n, 1, 1), (32, 1, 1), 0)
+
+
+class CoalescedGemvKernel(_GemvF32):
+    """gemv.rs:188-398: 256 threads per block, one output element per thread, x tiles of 256 in shared memory."""
+    _NAME = "gemv_coalesced"
+
+    def launch_config(self) -> LaunchConfig:
+        return LaunchConfig(((self.n + 255) // 256, 1, 1), (256, 1, 1), 1024)
