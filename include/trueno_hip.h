@@ -182,6 +182,12 @@ TRN_API trn_status trn_event_destroy(trn_event event);
 TRN_API trn_status trn_event_record(trn_event event, trn_stream stream);
 TRN_API trn_status trn_event_synchronize(trn_event event);
 TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop);
+/* Re-packs n_sb GGML Q5_K blocks (what a GGUF file holds: d, dmin, scales[12], qh[32], qs[128]) into the Q5_K
+ * layout of the reference's kernels (trueno-gpu/src/kernels/quantize.rs:1589-1693, which is not GGML's); the
+ * dequantised values are unchanged.  dst may be src.  Q4_K and Q6_K need no such step: the reference reads GGML's
+ * bytes as they are.  No counterpart in the reference: its callers re-pack on the host. */
+TRN_API trn_status trn_q5k_from_ggml(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t n_sb);
+
 /* f32 GEMV: y[n] = sum_k a[k*n_dim + n] * x[k]; a is K x N row-major, i.e. transposed relative to the quantized
  * matrices.  trueno-gpu/src/kernels/gemv.rs: GemvKernel "gemv_warp_reduce" :21-166 and CoalescedGemvKernel
  * "gemv_coalesced" :188-398, both (y_ptr, a_ptr, x_ptr, k_dim, n_dim); the built-in module has both names.  Keeps a

@@ -137,6 +137,46 @@ def dequant_q5k(buf) -> np.ndarray:
     return ((ds_v * q) - dm_v).astype(F32)
 
 
+def dequant_q5k_ggml(buf) -> np.ndarray:
+    """GGML's own Q5_K block (public format: block_q5_K = d, dmin, scales[12], qh[32], qs[128]; dequantize_row_q5_K):
+    scales/mins packed as in Q4_K (get_scale_min_k4); value i = 32 j + l has the nibble of qs[32 (i//64) + l] (low for
+    even j) and its fifth bit in bit j of qh[l];  w = (d*sc_j)*q - dmin*m_j.  NOT the reference's Q5_K layout - this
+    is what a GGUF file holds; q5k_ggml_to_reference() turns one into the other."""
+    blk = _as_blocks(buf, Q5K_BYTES)
+    d = _f16_at(blk, 0)
+    dmin = _f16_at(blk, 2)
+    s, m = scales_mins_k4(blk[:, 4:16])
+    qh = blk[:, 16:48].astype(np.uint32)
+    ql = _nibbles_chunked(blk[:, 48:176]).astype(np.uint32)
+    i = np.arange(256)
+    hb = (qh[:, i % 32] >> (i // 32)) & 1
+    q = (ql + 16 * hb).astype(F32)
+    ds_v = np.repeat(d[:, None] * s.astype(F32), 32, axis=1)
+    dm_v = np.repeat(dmin[:, None] * m.astype(F32), 32, axis=1)
+    return ((ds_v * q) - dm_v).astype(F32)
+
+
+def q5k_ggml_to_reference(buf) -> np.ndarray:
+    """Re-pack GGML Q5_K blocks into the layout decode B reads (quantize.rs:1589-1693): header kept, the eight
+    (scale, min) pairs as contiguous 12-bit fields, qs moved to offset 16, the fifth bits re-ordered so that value i
+    is bit i%8 of qh[i//8] at offset 144.  dequant_q5k(result) == dequant_q5k_ggml(input), bit for bit."""
+    blk = _as_blocks(buf, Q5K_BYTES)
+    out = np.zeros_like(blk)
+    out[:, 0:4] = blk[:, 0:4]
+    s, m = scales_mins_k4(blk[:, 4:16])
+    fields = (s.astype(np.uint64) | (m.astype(np.uint64) << np.uint64(6)))          # 12 bits each
+    bits = np.zeros((blk.shape[0], 96), np.uint8)
+    for j in range(8):
+        for r in range(12):
+            bits[:, 12 * j + r] = (fields[:, j] >> np.uint64(r)) & np.uint64(1)
+    out[:, 4:16] = np.packbits(bits, axis=1, bitorder="little")
+    out[:, 16:144] = blk[:, 48:176]
+    i = np.arange(256)
+    hb = ((blk[:, 16:48][:, i % 32] >> (i // 32)) & 1).astype(np.uint8)
+    out[:, 144:176] = np.packbits(hb, axis=1, bitorder="little")
+    return out.reshape(-1)
+
+
 def dequant_q6k(buf) -> np.ndarray:
     """Decode C.  Block: ql[128]@0 qh[64]@128 sc[16] int8 @192 d@208.
     value i: h=i//128, p=i%128, g=p//32, l=p%32; scale sc[8h + l//16 + 2g];

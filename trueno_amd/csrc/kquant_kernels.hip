@@ -153,6 +153,50 @@ extern "C" __global__ void __launch_bounds__(256) gemv_coalesced(float* y, const
   gemv_f32::generic_body(y, a, x, k_dim, n_dim);
 }
 
+// GGML's Q5_K block (d, dmin, scales[12] packed as in Q4_K, qh[32], qs[128]; fifth bit of value 32 j + l in bit j of
+// qh[l]) re-packed into the layout the reference's Q5_K kernels read (trueno-gpu/src/kernels/quantize.rs:1589-1693:
+// d, dmin, eight contiguous 12-bit (scale, min) fields, qs[128] at 16, fifth bit of value i in bit i%8 of qh[i/8]
+// at 144).  The dequantised values are the same, bit for bit.  One wave per block; dst may be src (a wave reads
+// its whole block before it writes).
+extern "C" __global__ void __launch_bounds__(256) q5k_from_ggml(uint8_t* dst, const uint8_t* src, uint64_t n_sb) {
+  const u32 lane = threadIdx.x & 63u;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  const uint64_t nwaves = (static_cast<uint64_t>(gridDim.x) * blockDim.x) >> 6;
+  for (uint64_t sb = wave; sb < n_sb; sb += nwaves) {
+    const uint8_t* in = src + sb * 176u;
+    uint8_t* out = dst + sb * 176u;
+    // everything this lane needs, before anything is written
+    const u32 hdr = lane < 4u ? in[lane] : 0u;
+    u32 sc[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) sc[i] = in[4 + i];
+    const u32 q0 = in[48u + 2u * lane], q1 = in[49u + 2u * lane];
+    u32 hb = 0u;                       // lanes 0..31: byte `lane` of the new qh = values 8 lane .. 8 lane + 7
+    if (lane < 32u) {
+      const u32 j = lane >> 2, l0 = 8u * (lane & 3u);
+#pragma unroll
+      for (u32 b = 0; b < 8; ++b) hb |= ((static_cast<u32>(in[16u + l0 + b]) >> j) & 1u) << b;
+    }
+    u32 fb = 0u;                       // lanes 0..11: byte `lane` of the 96-bit string of 12-bit fields
+    if (lane < 12u) {
+#pragma unroll
+      for (u32 b = 0; b < 8; ++b) {
+        const u32 p = 8u * lane + b, j = p / 12u, r = p % 12u;
+        u32 s6, m6;                    // get_scale_min_k4
+        if (j < 4u) { s6 = sc[j] & 63u; m6 = sc[j + 4] & 63u; }
+        else { s6 = (sc[j + 4] & 15u) | ((sc[j - 4] >> 6) << 4); m6 = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4); }
+        fb |= (((r < 6u ? s6 >> r : m6 >> (r - 6u))) & 1u) << b;
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane < 4u) out[lane] = static_cast<uint8_t>(hdr);
+    if (lane < 12u) out[4u + lane] = static_cast<uint8_t>(fb);
+    out[16u + 2u * lane] = static_cast<uint8_t>(q0);
+    out[17u + 2u * lane] = static_cast<uint8_t>(q1);
+    if (lane < 32u) out[144u + lane] = static_cast<uint8_t>(hb);
+  }
+}
+
 extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32 v) {
   for (u32 i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = v;
 }

@@ -67,7 +67,7 @@ struct DeviceKernels {
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
-  hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr;
+  hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr;
   hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
@@ -124,6 +124,7 @@ hipError_t device_kernels(DeviceKernels** out) {
     }
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_f32_fast, "gemv_f32_fast")) != hipSuccess ||
+        (e = get_fn(m, &t.q5k_from_ggml, "q5k_from_ggml")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_f32_generic, "gemv_coalesced")) != hipSuccess ||
         (e = get_fn(m, &t.residual_add, "residual_add")) != hipSuccess ||
         (e = get_fn(m, &t.swiglu, "fused_swiglu")) != hipSuccess ||
@@ -1080,6 +1081,15 @@ trn_status trn_q4k_simplified_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w
   return st(launch_dequant_simplified(static_cast<hipStream_t>(s), out, w, n_blocks));
 }
 
+trn_status trn_q5k_from_ggml(trn_stream s, trn_dptr dst, trn_dptr src, uint64_t n_sb) {
+  if (n_sb == 0) return TRN_SUCCESS;
+  if (!dst || !src) return TRN_ERROR_INVALID_VALUE;
+  DeviceKernels* d = nullptr;
+  TRN_TRY(device_kernels(&d));
+  const uint32_t grid = uint32_t(std::min<uint64_t>((n_sb + 3u) / 4u, uint64_t(d->cu_count) * 32u));
+  void* args[] = {&dst, &src, &n_sb};
+  return st(hipModuleLaunchKernel(d->q5k_from_ggml, grid, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(s), args, nullptr));
+}
 trn_status trn_gemv_f32(trn_stream s, trn_dptr y, trn_dptr a, trn_dptr x, uint32_t k, uint32_t n) {
   return st(launch_gemv_f32(static_cast<hipStream_t>(s), y, a, x, k, n));
 }
