@@ -344,6 +344,35 @@ def main() -> int:
             for b in bufs:
                 b.free()
 
+    # ---- single-query attention over a KV cache of 7B shape (32 heads x 128), one launch, cold ------------------
+    attention = {}
+    if not args.no_configs:
+        rng = np.random.default_rng(66)
+        heads, dim = 32, 128
+        for seq in (512, 2048, 8192):
+            copies = 6
+            kvs = [(t.GpuBuffer.from_host(ctx, rng.standard_normal(heads * seq * dim, dtype=np.float32)),
+                    t.GpuBuffer.from_host(ctx, rng.standard_normal(heads * seq * dim, dtype=np.float32))) for _ in range(copies)]
+            qb, ob = xs[0][0], y[4096]
+            def launch(r):
+                return L.trn_incremental_attention(stream.raw(), qb.as_ptr(), kvs[r % copies][0].as_ptr(), kvs[r % copies][1].as_ptr(),
+                                                   ob.as_ptr(), seq, dim, heads, heads, seq, C.c_float(dim ** -0.5))
+            for r in range(copies):
+                assert launch(r) == 0
+            stream.synchronize()
+            L.trn_event_record(e0, stream.raw())
+            for r in range(2 * copies):
+                launch(r)
+            L.trn_event_record(e1, stream.raw())
+            stream.synchronize()
+            us = elapsed_ms(e0, e1) * 1e3 / (2 * copies)
+            nbytes = 8 * heads * seq * dim + 8 * heads * dim
+            attention[f"seq{seq}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                      "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            for a, b in kvs:
+                a.free()
+                b.free()
+
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
     cpu_config1 = None
@@ -398,7 +427,7 @@ def main() -> int:
                   "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
                   "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": round(layer_ms * 1e3, 1),
-                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "f32_gemv_single_launch_cold": f32_gemv,
+                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "f32_gemv_single_launch_cold": f32_gemv, "incremental_attention_32x128_single_launch_cold": attention,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }

@@ -182,6 +182,18 @@ TRN_API trn_status trn_event_destroy(trn_event event);
 TRN_API trn_status trn_event_record(trn_event event, trn_stream stream);
 TRN_API trn_status trn_event_synchronize(trn_event event);
 TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop);
+/* Single-query attention over a KV cache, the step between the q/k/v and the o projection of a decoding layer:
+ *   out[h] = sum_i softmax_i(scale * q[h] . k[kv(h)][i]) v[kv(h)][i],  i < seq_len,  kv(h) = h * num_kv_heads / num_heads
+ *   q, out: [num_heads][head_dim] f32;  k, v: [num_kv_heads][max_seq_len][head_dim] f32.
+ * trueno-gpu/src/kernels/attention.rs:808-1095 (IncrementalAttentionKernel, "incremental_attention", parameters
+ * (q_ptr, k_ptr, v_ptr, out_ptr, seq_len); head_dim, the head counts, max_seq_len and scale are compiled into its
+ * PTX and follow as parameters here, also in a by-name launch).  The reference's kernel covers head_dim <= 64;
+ * this one head_dim % 4 == 0 up to 256.  1 <= seq_len <= max_seq_len; pointers 16-byte aligned.  Keeps a small
+ * per-stream workspace (allocated on first use). */
+TRN_API trn_status trn_incremental_attention(trn_stream stream, trn_dptr q, trn_dptr k, trn_dptr v, trn_dptr out,
+                                             uint32_t seq_len, uint32_t head_dim, uint32_t num_heads, uint32_t num_kv_heads,
+                                             uint32_t max_seq_len, float scale);
+
 /* Re-packs n_sb GGML Q5_K blocks (what a GGUF file holds: d, dmin, scales[12], qh[32], qs[128]) into the Q5_K
  * layout of the reference's kernels (trueno-gpu/src/kernels/quantize.rs:1589-1693, which is not GGML's); the
  * dequantised values are unchanged.  dst may be src.  Q4_K and Q6_K need no such step: the reference reads GGML's

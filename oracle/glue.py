@@ -11,6 +11,7 @@ Reference lines followed (under trueno-gpu/src/kernels/):
   gemv_warp_reduce        gemv.rs:21-166           y[n] = sum_k A[k][n] x[k], A K x N row-major; lane t of 32 takes
                                                    k = t, t+32, ... by fma, then the shfl.down tree
   gemv_coalesced          gemv.rs:188-398          the same product, one thread per column, k in order by fma
+  incremental_attention   attention.rs:808-1095    one query per head over a KV cache, online softmax position by position
 (div.f32 is printed as div.rn, ex2/rsqrt as .approx: trueno-gpu/src/ptx/builder.rs:1425-1431, 1523-1530.)
 
 Every f32 operation is rounded separately, as the reference's instructions are.  The two approximate
@@ -27,6 +28,9 @@ How each function is pinned (the reference holds no numeric test of these kernel
                           agreement with the fp64 formula; the lane order is an emulation used for error magnitudes.
   gemv_f32_*            : an fp64 matrix product is the closed form; brute force on tiny shapes; the two f32 orders
                           are emulations used for error magnitudes only.
+  incremental_attention : fp64 softmax attention is the closed form; special cases (one position; equal keys give the
+                          mean of the values; one dominant key gives its value); the position-by-position f32 recurrence
+                          is an emulation used for error magnitudes only.
 Against a running reference these stay "parity unpinned": it cannot be run here (no Rust, no NVIDIA driver).
 """
 import numpy as np
@@ -124,3 +128,45 @@ def gemv_f32_warp_reduce_order(a, x):
         nxt[:32 - d] = (lanes[:32 - d] + lanes[d:]).astype(F32)
         lanes = nxt
     return lanes[0]
+
+
+def attention_fp64(q, k, v, seq_len, scale=None):
+    """out[h] = softmax(scale * q[h] . k[kv(h)][:seq_len]) @ v[kv(h)][:seq_len], kv(h) = h * num_kv_heads // num_heads
+    (attention.rs:877-885, 920-922).  q [H][D]; k, v [Hkv][max_seq][D]."""
+    q, k, v = (np.asarray(a, np.float64) for a in (q, k, v))
+    H, D = q.shape
+    Hkv = k.shape[0]
+    scale = 1.0 / np.sqrt(D) if scale is None else float(scale)
+    out = np.zeros((H, D))
+    for h in range(H):
+        kv = h * Hkv // H
+        s = (k[kv, :seq_len] @ q[h]) * scale
+        w = np.exp(s - s.max())
+        out[h] = (w / w.sum()) @ v[kv, :seq_len]
+    return out
+
+
+def attention_ref_order(q, k, v, seq_len, scale=None):
+    """The reference's recurrence in f32 (attention.rs:963-1066): per position the dot product (lane order ignored:
+    summed in f64 and rounded once), score = dot * scale, new max, correction = 2^((old-new)*log2e), e = 2^((score-new)*log2e),
+    sum = sum*correction + e, out = out*correction + e*v; finally out * (1/sum).  ex2 evaluated exactly."""
+    q, k, v = (np.asarray(a, F32) for a in (q, k, v))
+    H, D = q.shape
+    Hkv = k.shape[0]
+    scale = F32(1.0 / np.sqrt(F32(D))) if scale is None else F32(scale)
+    log2e = F32(1.4426950)
+    out = np.zeros((H, D), F32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        for h in range(H):
+            kv = h * Hkv // H
+            m, ssum, o = F32(-np.inf), F32(0.0), np.zeros(D, F32)
+            for p in range(seq_len):
+                score = F32(F32(np.dot(q[h].astype(np.float64), k[kv, p].astype(np.float64))) * scale)
+                nm = max(m, score)
+                corr = F32(np.exp2(np.float64(F32(F32(m - nm) * log2e)))) if np.isfinite(m) else F32(0.0)
+                e = F32(np.exp2(np.float64(F32(F32(score - nm) * log2e))))
+                ssum = F32(F32(ssum * corr) + e)
+                o = ((o * corr).astype(F32).astype(np.float64) + np.float64(e) * v[kv, p].astype(np.float64)).astype(F32)
+                m = nm
+            out[h] = (o * F32(F32(1.0) / ssum)).astype(F32)
+    return out

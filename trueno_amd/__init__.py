@@ -8,7 +8,8 @@ over the C ABI of libtrueno_hip.so:
     trueno_amd.kernels  Kernel, Q4KGemvKernel, Q5KGemvKernel, Q6KGemvKernel, QuantizeKernel,
                         Q5KKernel, Q6KKernel, Q4KFormat   (trueno-gpu/src/kernels/quantize.rs)
     trueno_amd.glue     ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel, GemvKernel,
-                        CoalescedGemvKernel   (trueno-gpu/src/kernels/elementwise.rs, layernorm.rs, gemv.rs)
+                        CoalescedGemvKernel, IncrementalAttentionKernel
+                        (trueno-gpu/src/kernels/elementwise.rs, layernorm.rs, gemv.rs, attention.rs)
 
 There is no CPU path: without libtrueno_hip.so or without a GPU every device call raises GpuError.
 """
@@ -18,4 +19,4 @@ from .driver import (CudaContext, CudaModule, CudaStream, GpuBuffer, GpuError, L
 from .kernels import (GemvBatch, Kernel, Q4KFormat, Q4KGemvKernel, Q5KGemvKernel, Q5KKernel, Q6KGemvKernel,  # noqa: F401
                       Q6KKernel, QuantizeKernel)
 from .glue import (CoalescedGemvKernel, FusedResidualRmsNormKernel, FusedSwigluKernel, GemvKernel,  # noqa: F401
-                   ResidualAddKernel, RmsNormKernel)
+                   IncrementalAttentionKernel, ResidualAddKernel, RmsNormKernel)

@@ -51,6 +51,7 @@ SIGNATURES = {
     "trn_q4k_gemm_fused": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_gemv_f32": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32],
     "trn_q5k_from_ggml": [vp, dptr, dptr, C.c_uint64],
+    "trn_incremental_attention": [vp, dptr, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_float],
     "trn_residual_add": [vp, dptr, dptr, dptr, C.c_uint32],
     "trn_fused_swiglu": [vp, dptr, dptr, dptr, C.c_uint32],
     "trn_rmsnorm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_float],

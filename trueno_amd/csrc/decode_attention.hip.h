@@ -1,0 +1,133 @@
+// Single-query attention over a KV cache for autoregressive decoding (trueno-gpu/src/kernels/attention.rs:808-1095,
+// IncrementalAttentionKernel, kernel name "incremental_attention"):
+//   out[h][:] = sum_i softmax_i(scale * q[h] . k[kv(h)][i]) * v[kv(h)][i],  i < seq_len,  kv(h) = h * num_kv_heads / num_heads
+//   q, out: [num_heads][head_dim];  k, v: [num_kv_heads][max_seq_len][head_dim];  f32.
+// The reference walks the positions one by one in a single warp per head with an online softmax (Milakov &
+// Gimelshein) and two elements per lane, which covers head_dim <= 64; this kernel computes the same function for
+// head_dim up to 256.  Bound by HBM: K and V are read once, 8 * num_kv_heads * seq_len * head_dim bytes.
+//
+// A position's row of K (and of V) is read by head_dim/4 lanes with one 128-bit load each, so a wave takes
+// 64 / (head_dim/4) positions at a time; each such lane group keeps its own running (max, sum, output) over the
+// positions it sees.  The positions of a head are cut in chunks over the grid and a chunk over the 4 waves of a
+// workgroup; groups, waves and chunks are merged with the usual rescaling, the chunks through memory by the
+// workgroup that arrives last at the head's counter (in chunk order: the same bits on every run).  Exponentials
+// are 2^x on scores pre-multiplied by log2(e), as in the reference (ex2.approx there, v_exp_f32 here).
+#pragma once
+#include "kquant_common.hip.h"
+
+namespace decode_attention {
+
+constexpr u32 kWaves = 4;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct State {          // running softmax over some positions, in the 2^x domain
+  float m, s;
+  f32x4 o;
+};
+
+__device__ __forceinline__ void merge(State& a, float m, float s, const f32x4& o) {
+  const float nm = fmaxf(a.m, m);
+  const float ca = a.m == nm ? 1.0f : __builtin_amdgcn_exp2f(a.m - nm);     // -inf - -inf never reaches exp2
+  const float cb = m == nm ? 1.0f : __builtin_amdgcn_exp2f(m - nm);
+  a.s = a.s * ca + s * cb;
+  a.o.x = a.o.x * ca + o.x * cb; a.o.y = a.o.y * ca + o.y * cb;
+  a.o.z = a.o.z * ca + o.z * cb; a.o.w = a.o.w * ca + o.w * cb;
+  a.m = nm;
+}
+
+// lanes per position LPP = 2^lpp_log2 >= head_dim / 4
+__device__ __forceinline__ void body(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                     float* __restrict__ out, u32 seq_len, u32 head_dim, u32 num_heads, u32 num_kv_heads,
+                                     u32 max_seq_len, float scale, u32 lpp_log2, u32 chunk, u32 chunks,
+                                     float* __restrict__ partial, u32* __restrict__ counters) {
+  __shared__ float s_m[kWaves][64], s_s[kWaves][64];
+  __shared__ f32x4 s_o[kWaves][64];
+  __shared__ u32 s_old;
+  const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const u32 head = blockIdx.x / chunks, ci = blockIdx.x - head * chunks;
+  const u32 kv_head = static_cast<u32>((static_cast<uint64_t>(head) * num_kv_heads) / num_heads);
+  const u32 lpp = 1u << lpp_log2, ppw = 64u >> lpp_log2;           // lanes per position, positions per wave and step
+  const u32 sub = lane & (lpp - 1u), grp = lane >> lpp_log2;
+  const bool live = 4u * sub < head_dim;                             // head_dim % 4 == 0
+  const size_t kv_base = static_cast<size_t>(kv_head) * max_seq_len * head_dim;
+  const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f32x4 qv = live ? reinterpret_cast<const f32x4*>(q + static_cast<size_t>(head) * head_dim)[sub] : zero4;
+  const float sl = scale * kLog2e;
+  const u32 p0 = ci * chunk, p1 = min(seq_len, p0 + chunk);
+  State st = {-INFINITY, 0.0f, zero4};
+  constexpr u32 kAhead = 4;                     // positions per lane group whose rows are in flight together
+  const u32 stride = kWaves * ppw;
+  for (u32 p = p0 + wave * ppw + grp; p < p1; p += kAhead * stride) {
+    f32x4 kk[kAhead], vv[kAhead];
+#pragma unroll
+    for (u32 a = 0; a < kAhead; ++a) {
+      const u32 pa = min(p + a * stride, p1 - 1u);          // clamped: read, then ignored
+      const size_t row = kv_base + static_cast<size_t>(pa) * head_dim;
+      kk[a] = live ? reinterpret_cast<const f32x4*>(k + row)[sub] : zero4;
+      vv[a] = live ? reinterpret_cast<const f32x4*>(v + row)[sub] : zero4;
+    }
+#pragma unroll
+    for (u32 a = 0; a < kAhead; ++a) {
+      float d = fmaf(qv.w, kk[a].w, fmaf(qv.z, kk[a].z, fmaf(qv.y, kk[a].y, qv.x * kk[a].x)));
+      for (u32 off = 1; off < lpp; off <<= 1) d += __shfl_xor(d, off, 64);        // within the lane group
+      if (p + a * stride < p1) merge(st, d * sl, 1.0f, vv[a]);
+    }
+  }
+  // the lane groups of a wave, then the waves of the workgroup: lane `sub` of group 0 ends up with the chunk's state
+  for (u32 off = lpp; off < 64u; off <<= 1) {
+    const float m = __shfl_xor(st.m, off, 64), s = __shfl_xor(st.s, off, 64);
+    f32x4 o;
+    o.x = __shfl_xor(st.o.x, off, 64); o.y = __shfl_xor(st.o.y, off, 64);
+    o.z = __shfl_xor(st.o.z, off, 64); o.w = __shfl_xor(st.o.w, off, 64);
+    merge(st, m, s, o);
+  }
+  s_m[wave][lane] = st.m; s_s[wave][lane] = st.s; s_o[wave][lane] = st.o;
+  __syncthreads();
+  if (wave != 0u || lane >= lpp) {
+    if (chunks == 1u) return;
+  } else {
+    for (u32 w = 1; w < kWaves; ++w) merge(st, s_m[w][lane], s_s[w][lane], s_o[w][lane]);
+    float* dst = out + static_cast<size_t>(head) * head_dim + 4u * sub;
+    if (chunks == 1u) {
+      if (live) {
+        const float inv = 1.0f / st.s;
+        *reinterpret_cast<f32x4*>(dst) = f32x4{st.o.x * inv, st.o.y * inv, st.o.z * inv, st.o.w * inv};
+      }
+      return;
+    }
+    // [head][chunk][lpp lanes][m, s, o.xyzw] through to memory
+    u32* pp = reinterpret_cast<u32*>(partial) + ((static_cast<size_t>(head) * chunks + ci) * lpp + sub) * 8u;
+    const float vals[6] = {st.m, st.s, st.o.x, st.o.y, st.o.z, st.o.w};
+#pragma unroll
+    for (int i = 0; i < 6; ++i) __hip_atomic_store(pp + i, __float_as_uint(vals[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0u) {
+      const u32 old = __hip_atomic_fetch_add(counters + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (old == chunks - 1u) __hip_atomic_store(counters + head, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_old = old;
+    }
+  }
+  __syncthreads();
+  if (wave != 0u || lane >= lpp || s_old != chunks - 1u) return;
+  State tot = {-INFINITY, 0.0f, zero4};
+  for (u32 c0 = 0; c0 < chunks; c0 += 8u) {        // eight chunks' states in flight, merged in chunk order
+    float vals[8][6];
+#pragma unroll
+    for (u32 cc = 0; cc < 8; ++cc) {
+      const u32 c = min(c0 + cc, chunks - 1u);
+      const u32* pp = reinterpret_cast<const u32*>(partial) + ((static_cast<size_t>(head) * chunks + c) * lpp + sub) * 8u;
+#pragma unroll
+      for (int i = 0; i < 6; ++i) vals[cc][i] = __uint_as_float(__hip_atomic_load(pp + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    }
+#pragma unroll
+    for (u32 cc = 0; cc < 8; ++cc)
+      if (c0 + cc < chunks) merge(tot, vals[cc][0], vals[cc][1], f32x4{vals[cc][2], vals[cc][3], vals[cc][4], vals[cc][5]});
+  }
+  if (live) {
+    const float inv = 1.0f / tot.s;
+    *reinterpret_cast<f32x4*>(out + static_cast<size_t>(head) * head_dim + 4u * sub) =
+        f32x4{tot.o.x * inv, tot.o.y * inv, tot.o.z * inv, tot.o.w * inv};
+  }
+}
+
+}  // namespace decode_attention

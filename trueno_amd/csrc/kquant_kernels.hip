@@ -13,6 +13,7 @@
 #include "kquant_gemm_f16.hip.h"
 #include "decode_glue.hip.h"
 #include "gemv_f32.hip.h"
+#include "decode_attention.hip.h"
 
 // The fast GEMV engine is chain_step() of kquant_chain.hip.h: one workgroup owns a run of rows; the
 // activation vector is staged once into LDS (swizzled), each wave keeps its 64-activations-per-lane
@@ -195,6 +196,17 @@ extern "C" __global__ void __launch_bounds__(256) q5k_from_ggml(uint8_t* dst, co
     out[17u + 2u * lane] = static_cast<uint8_t>(q1);
     if (lane < 32u) out[144u + lane] = static_cast<uint8_t>(hb);
   }
+}
+
+// Single-query attention over the KV cache (decode_attention.hip.h) under the reference's kernel name.  The reference's
+// parameter list is (q_ptr, k_ptr, v_ptr, out_ptr, seq_len) with head_dim, the head counts, max_seq_len and the scale
+// compiled into the PTX (attention.rs:865-901); here they follow as parameters, then the launcher's own.
+extern "C" __global__ void __launch_bounds__(256)
+incremental_attention(const float* q, const float* k, const float* v, float* out, u32 seq_len, u32 head_dim, u32 num_heads,
+                      u32 num_kv_heads, u32 max_seq_len, float scale, u32 lpp_log2, u32 chunk, u32 chunks, float* partial,
+                      u32* counters) {
+  decode_attention::body(q, k, v, out, seq_len, head_dim, num_heads, num_kv_heads, max_seq_len, scale, lpp_log2, chunk, chunks,
+                         partial, counters);
 }
 
 extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32 v) {

@@ -44,7 +44,7 @@ const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 
 // kinds of functions the launch-by-name path recognises
 enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3, KIND_RESIDUAL_ADD = 4, KIND_SWIGLU = 5,
-            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8 };
+            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8, KIND_ATTENTION = 9 };
 
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
@@ -67,7 +67,7 @@ struct DeviceKernels {
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
-  hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr;
+  hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
   hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
@@ -125,6 +125,7 @@ hipError_t device_kernels(DeviceKernels** out) {
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_f32_fast, "gemv_f32_fast")) != hipSuccess ||
         (e = get_fn(m, &t.q5k_from_ggml, "q5k_from_ggml")) != hipSuccess ||
+        (e = get_fn(m, &t.attention, "incremental_attention")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_f32_generic, "gemv_coalesced")) != hipSuccess ||
         (e = get_fn(m, &t.residual_add, "residual_add")) != hipSuccess ||
         (e = get_fn(m, &t.swiglu, "fused_swiglu")) != hipSuccess ||
@@ -281,6 +282,54 @@ hipError_t launch_gemv_f32(hipStream_t stream, uint64_t y, uint64_t a, uint64_t 
   uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
   void* args[] = {&y, &a, &x, &part, &cnt, &k, &n, &rows_per_part, &parts};
   return hipModuleLaunchKernel(d->gemv_f32_fast, tiles * parts, 1, 1, 512, 1, 1, 0, stream, args, nullptr);
+}
+
+// Single-query attention over the KV cache (decode_attention.hip.h).  Per (device, stream): arrival counters per
+// head and the chunks' partial softmax states.
+std::map<std::pair<int, hipStream_t>, GemvF32Workspace> g_attention_ws;
+
+hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t v, uint64_t out, uint32_t seq_len,
+                            uint32_t head_dim, uint32_t num_heads, uint32_t num_kv_heads, uint32_t max_seq_len, float scale) {
+  if (num_heads == 0) return hipSuccess;
+  if (!q || !k || !v || !out || seq_len == 0 || seq_len > max_seq_len || head_dim == 0 || head_dim % 4u != 0 || head_dim > 256u ||
+      num_kv_heads == 0 || num_kv_heads > num_heads || num_heads > 16384u || !aligned(q, 16) || !aligned(k, 16) ||
+      !aligned(v, 16) || !aligned(out, 16))
+    return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  uint32_t lpp_log2 = 0;
+  while ((4u << lpp_log2) < head_dim) ++lpp_log2;
+  const uint32_t lpp = 1u << lpp_log2, step = 4u * (64u >> lpp_log2);       // positions a workgroup takes at a time
+  // chunks of positions per head: about two workgroups per CU, at least four steps each
+  uint32_t chunks = std::max(1u, (2u * uint32_t(d->cu_count) + num_heads - 1u) / num_heads);
+  chunks = std::max(1u, std::min(chunks, (seq_len + 4u * step - 1u) / (4u * step)));
+  uint32_t chunk = (seq_len + chunks - 1u) / chunks;
+  chunk = (chunk + step - 1u) / step * step;
+  chunks = (seq_len + chunk - 1u) / chunk;
+  const size_t cnt_cap = 64u * 1024u, need = cnt_cap + (chunks > 1u ? size_t(num_heads) * chunks * lpp * 32u : 0u);
+  int dev = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+  GemvF32Workspace* ws;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    ws = &g_attention_ws[std::make_pair(dev, stream)];
+  }
+  if (ws->cap < need) {
+    if (ws->buf) {
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;
+      (void)hipFree(ws->buf);
+      ws->buf = nullptr;
+      ws->cap = 0;
+    }
+    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
+    ws->cap = need;
+    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;   // the kernel leaves the counters at zero
+  }
+  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  void* args[] = {&q, &k, &v, &out, &seq_len, &head_dim, &num_heads, &num_kv_heads, &max_seq_len, &scale, &lpp_log2, &chunk, &chunks,
+                  &part, &cnt};
+  return hipModuleLaunchKernel(d->attention, num_heads * chunks, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
 }
 
 // Partial results and arrival counters of the matrix-core GEMM: one buffer per (device, stream), grown on
@@ -850,6 +899,7 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
     }
     if (n == "q4k_gemm_fused") h->kind = KIND_GEMM_SIMPLIFIED;
     if (n == "gemv_warp_reduce" || n == "gemv_coalesced") h->kind = KIND_GEMV_F32;
+    if (n == "incremental_attention") h->kind = KIND_ATTENTION;
     if (n == "residual_add") h->kind = KIND_RESIDUAL_ADD;
     if (n == "fused_swiglu") h->kind = KIND_SWIGLU;
     if (n == "rmsnorm") h->kind = KIND_RMSNORM;
@@ -959,6 +1009,18 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     std::memcpy(&k, kernel_params[5], 4);
     if (func->kind == KIND_GEMM_SIMPLIFIED) return st(launch_gemm_simplified(s, p0, p1, p2, m, n, k));
     return st(launch_gemm_like(Fmt(func->fmt), s, p0, p1, p2, m, n, k, false));
+  }
+  if (func->kind == KIND_ATTENTION) {      // (q, k, v, out, seq_len), then head_dim, num_heads, num_kv_heads, max_seq_len, scale
+    if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
+    for (int i = 0; i < 10; ++i)
+      if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
+    uint64_t p[4];
+    uint32_t u[5];
+    float scale;
+    for (int i = 0; i < 4; ++i) std::memcpy(&p[i], kernel_params[i], 8);
+    for (int i = 0; i < 5; ++i) std::memcpy(&u[i], kernel_params[4 + i], 4);
+    std::memcpy(&scale, kernel_params[9], 4);
+    return st(launch_attention(s, p[0], p[1], p[2], p[3], u[0], u[1], u[2], u[3], u[4], scale));
   }
   if (func->kind == KIND_GEMV_F32) {                                           // (y, a, x, k_dim, n_dim)
     if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
@@ -1081,6 +1143,10 @@ trn_status trn_q4k_simplified_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w
   return st(launch_dequant_simplified(static_cast<hipStream_t>(s), out, w, n_blocks));
 }
 
+trn_status trn_incremental_attention(trn_stream s, trn_dptr q, trn_dptr k, trn_dptr v, trn_dptr out, uint32_t seq_len,
+                                     uint32_t head_dim, uint32_t num_heads, uint32_t num_kv_heads, uint32_t max_seq_len, float scale) {
+  return st(launch_attention(static_cast<hipStream_t>(s), q, k, v, out, seq_len, head_dim, num_heads, num_kv_heads, max_seq_len, scale));
+}
 trn_status trn_q5k_from_ggml(trn_stream s, trn_dptr dst, trn_dptr src, uint64_t n_sb) {
   if (n_sb == 0) return TRN_SUCCESS;
   if (!dst || !src) return TRN_ERROR_INVALID_VALUE;

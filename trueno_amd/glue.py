@@ -158,3 +158,43 @@ class CoalescedGemvKernel(_GemvF32):
 
     def launch_config(self) -> LaunchConfig:
         return LaunchConfig(((self.n + 255) // 256, 1, 1), (256, 1, 1), 1024)
+
+
+class IncrementalAttentionKernel(Kernel):
+    """Single-query attention over a KV cache (attention.rs:808-1095): q, out [num_heads][head_dim];
+    k, v [num_kv_heads][max_seq_len][head_dim]."""
+
+    def __init__(self, max_seq_len: int, head_dim: int, num_heads: int):
+        self.max_seq_len, self.head_dim, self.num_heads = int(max_seq_len), int(head_dim), int(num_heads)
+        self.num_kv_heads = self.num_heads
+        self.scale = 1.0 / float(self.head_dim) ** 0.5           # attention.rs:849
+
+    @classmethod
+    def with_gqa(cls, max_seq_len: int, head_dim: int, num_heads: int, num_kv_heads: int) -> "IncrementalAttentionKernel":
+        k = cls(max_seq_len, head_dim, num_heads)
+        k.num_kv_heads = int(num_kv_heads)
+        return k
+
+    def is_gqa(self) -> bool:
+        return self.num_kv_heads != self.num_heads
+
+    def name(self) -> str:
+        return "incremental_attention"
+
+    def launch_config(self) -> LaunchConfig:
+        """one warp per query head (attention.rs:871-873)."""
+        return LaunchConfig((self.num_heads, 1, 1), (32, 1, 1), 0)
+
+    def kernel_args(self, q, k, v, out, seq_len: int):
+        """(q_ptr, k_ptr, v_ptr, out_ptr, seq_len) - attention.rs:897-901 - then what the reference compiles in."""
+        return [C.c_uint64(_ptr(q)), C.c_uint64(_ptr(k)), C.c_uint64(_ptr(v)), C.c_uint64(_ptr(out)), C.c_uint32(seq_len),
+                C.c_uint32(self.head_dim), C.c_uint32(self.num_heads), C.c_uint32(self.num_kv_heads),
+                C.c_uint32(self.max_seq_len), C.c_float(self.scale)]
+
+    def launch(self, stream: CudaStream, q, k, v, out, seq_len: int) -> None:
+        _check(_lib().trn_incremental_attention(stream.raw() if stream is not None else None, _ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                                int(seq_len), self.head_dim, self.num_heads, self.num_kv_heads, self.max_seq_len,
+                                                self.scale), "KernelLaunch", self.name())
+
+    def launch_by_name(self, stream: CudaStream, module: CudaModule, q, k, v, out, seq_len: int) -> None:
+        stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(q, k, v, out, seq_len))
