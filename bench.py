@@ -56,8 +56,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path runs on one GPU; --gpus must be 1 (a multi-GPU run would shard W by rows, "
-              "see DESIGN.md)", file=sys.stderr)
+        print("bench.py: this path runs on one GPU; --gpus must be 1 (several GPUs would each take a range of rows of "
+              "every matrix and exchange the output vectors)", file=sys.stderr)
         return 2
 
     import trueno_amd as t
