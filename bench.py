@@ -373,6 +373,51 @@ def main() -> int:
                 a.free()
                 b.free()
 
+    # ---- a whole decode step: the serial layer chain with folded glue AND attention over a KV cache of 2048 -------
+    decode_step = None
+    if not args.no_configs:
+        heads, dim, seq = 32, 128, 2048
+        rng = np.random.default_rng(77)
+        kv_host = rng.standard_normal(heads * seq * dim, dtype=np.float32)
+        caches = [(t.GpuBuffer.from_host(ctx, kv_host), t.GpuBuffer.from_host(ctx, kv_host)) for _ in range(layers)]
+        h0, h1 = t.GpuBuffer.from_host(ctx, kq.gen_x(778, 4096)), t.GpuBuffer(ctx, 4096, np.float32)
+        gam = t.GpuBuffer.from_host(ctx, np.abs(kq.gen_x(779, 4096)) + np.float32(0.5))
+        attn_out = t.GpuBuffer(ctx, 4096, np.float32)
+        pre, post = [], []
+        for layer in range(layers):
+            a, b = t.GemvBatch(), t.GemvBatch()
+            for name in ("q", "k", "v"):
+                a.add("q4k", 4096, 4096, act[name], weights[layer][name], h0, NORM, gamma=gam, norm_eps=1e-5)
+            b.add("q4k", 4096, 4096, h1, weights[layer]["o"], attn_out, 0, residual=h0)
+            for name in ("gate", "up"):
+                b.add("q4k", 4096, 11008, act[name], weights[layer][name], h1, NORM, gamma=gam, norm_eps=1e-5)
+            b.add("q6k", 11008, 4096, h0, weights[layer]["down"], act["gate"], 0, x2=act["up"], residual=h1)
+            pre.append(a)
+            post.append(b)
+        head_b = t.GemvBatch().add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, h0, NORM, gamma=gam, norm_eps=1e-5)
+
+        def step():
+            for layer in range(layers):
+                pre[layer].launch(stream)
+                L.trn_incremental_attention(stream.raw(), act["q"].as_ptr(), caches[layer][0].as_ptr(), caches[layer][1].as_ptr(),
+                                            attn_out.as_ptr(), seq, dim, heads, heads, seq, C.c_float(dim ** -0.5))
+                post[layer].launch(stream)
+            head_b.launch(stream)
+        step()
+        stream.synchronize()
+        L.trn_event_record(e0, stream.raw())
+        for _ in range(3):
+            step()
+        L.trn_event_record(e1, stream.raw())
+        stream.synchronize()
+        us = elapsed_ms(e0, e1) * 1e3 / 3
+        kv_bytes = layers * (8 * heads * seq * dim)
+        decode_step = {"us": round(us, 1), "kv_positions": seq, "weight_bytes": weight_bytes, "kv_cache_bytes": kv_bytes,
+                       "gbps": round((total_bytes + kv_bytes) / us / 1e3, 1)}
+        for a, b in caches:
+            a.free()
+            b.free()
+
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
     cpu_config1 = None
@@ -427,7 +472,7 @@ def main() -> int:
                   "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
                   "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": round(layer_ms * 1e3, 1),
-                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "f32_gemv_single_launch_cold": f32_gemv, "incremental_attention_32x128_single_launch_cold": attention,
+                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "decode_step_7b_folded_glue_and_attention": decode_step, "f32_gemv_single_launch_cold": f32_gemv, "incremental_attention_32x128_single_launch_cold": attention,
                   "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
                   "device": ctx.device_name(), "cus": ctx.cu_count()},
     }
