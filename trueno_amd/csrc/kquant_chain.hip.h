@@ -159,28 +159,25 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   const u32 units = k_dim >> 2;
   const u32 xgroups = units >> 6;                       // groups of 64 units; k is a multiple of 256
   const f32x4* x4 = reinterpret_cast<const f32x4*>(e.x);
+  // Across workgroups of one launch the vector is read past the (per-XCD, mutually incoherent) L2s: 16-byte
+  // buffer loads at agent scope (sc1), which the compiler tracks like any other load.
+  [[maybe_unused]] __amdgpu_buffer_rsrc_t x_rsrc, x2_rsrc;
+  if constexpr (COHERENT) {
+    x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(e.x), 0, static_cast<int>(k_dim * 4u), 0x00020000);
+    x2_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(e.x2 ? e.x2 : e.x), 0, static_cast<int>(k_dim * 4u), 0x00020000);
+  }
+  auto coherent16 = [](__amdgpu_buffer_rsrc_t r, u32 unit) {
+    const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(16u * unit), 0, 16 /* sc1 */);
+    return f32x4{__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w)};
+  };
   auto load_x = [&](u32 u) {
     f32x4 v;
-    if constexpr (COHERENT) {
-      const u32* xw = reinterpret_cast<const u32*>(e.x) + 4u * u;
-      v.x = __uint_as_float(__hip_atomic_load(xw + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      v.y = __uint_as_float(__hip_atomic_load(xw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      v.z = __uint_as_float(__hip_atomic_load(xw + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      v.w = __uint_as_float(__hip_atomic_load(xw + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    } else {
-      v = x4[u];
-    }
+    if constexpr (COHERENT) v = coherent16(x_rsrc, u);
+    else v = x4[u];
     if (e.flags & CHAIN_SWIGLU_INPUT) {
       f32x4 g2;
-      if constexpr (COHERENT) {
-        const u32* xw = reinterpret_cast<const u32*>(e.x2) + 4u * u;
-        g2.x = __uint_as_float(__hip_atomic_load(xw + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        g2.y = __uint_as_float(__hip_atomic_load(xw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        g2.z = __uint_as_float(__hip_atomic_load(xw + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        g2.w = __uint_as_float(__hip_atomic_load(xw + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      } else {
-        g2 = reinterpret_cast<const f32x4*>(e.x2)[u];
-      }
+      if constexpr (COHERENT) g2 = coherent16(x2_rsrc, u);
+      else g2 = reinterpret_cast<const f32x4*>(e.x2)[u];
       v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
     }
     return v;

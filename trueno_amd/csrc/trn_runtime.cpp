@@ -537,7 +537,9 @@ hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t strea
     double total = 0.0;
     std::vector<double> bytes(m);
     for (uint32_t i = 0; i < m; ++i) {
-      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4];
+      // cost, not bytes: a Q6_K byte takes longer than a Q4_K byte (measured: the workgroups of a Q6_K entry with
+      // a byte share ended 5 us after those of its Q4_K neighbours)
+      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4] * (descs[a + i].fmt == 6 ? 1.3 : 1.0);
       total += bytes[i];
     }
     // shares: at least one workgroup each, the rest in proportion to the bytes (largest remainders first)
@@ -557,7 +559,9 @@ hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t strea
     for (uint32_t i = 0; i < m; ++i) {
       const trn_gemv_desc& e = descs[a + i];
       const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, kWaves), groups = kWaves / sw;
-      const uint32_t ug = kGemvRowsPerBatch * groups;
+      // 12 waves hand their row batches out among themselves: a share need not be a whole number of rounds
+      const uint32_t ug = kGemvRowsPerBatch;
+      (void)groups;
       uint64_t rows = (uint64_t(e.n) + share[i] - 1) / share[i];
       rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
       const uint64_t need = uint64_t(e.k) * 4u + uint64_t(sw) * rows * 4u + kLdsScratch;
