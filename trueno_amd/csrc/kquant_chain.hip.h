@@ -195,9 +195,13 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   // in flight across the barrier and the activation staging.  Issued by every wave, also one without rows
   // (it reads clamped, valid addresses and ignores them): a branch here would hide the number of loads in
   // flight from the compiler, which then waits for all of them before the first activation is staged.
-  issue(sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
+  // The wave that polls a barrier asks for its rows only when the barrier has opened: loads return in order, and the
+  // answer to a poll behind weight loads comes late, for the whole workgroup.
+  const bool polls = wait_counter != nullptr && wave == 0u;
+  if (!polls) issue(sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
 
   if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
+  if (polls) issue(sw, wave_active ? grp : 0u);
   CHAIN_STAMP(1);
   if (!has_rows) return true;
 
