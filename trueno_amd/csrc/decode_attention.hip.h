@@ -51,6 +51,9 @@ __device__ __forceinline__ void body(const float* __restrict__ q, const float* _
   const bool live = 4u * sub < head_dim;                             // head_dim % 4 == 0
   const size_t kv_base = static_cast<size_t>(kv_head) * max_seq_len * head_dim;
   const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+  // the chunks' states cross workgroups (and XCDs): 16-byte buffer accesses at agent scope (sc1)
+  const __amdgpu_buffer_rsrc_t part_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(partial, 0, static_cast<int>(min(static_cast<size_t>(0x7FFFFFFF), static_cast<size_t>(num_heads) * chunks * lpp * 32u)), 0x00020000);
   const f32x4 qv = live ? reinterpret_cast<const f32x4*>(q + static_cast<size_t>(head) * head_dim)[sub] : zero4;
   const float sl = scale * kLog2e;
   const u32 p0 = ci * chunk, p1 = min(seq_len, p0 + chunk);
@@ -95,11 +98,11 @@ __device__ __forceinline__ void body(const float* __restrict__ q, const float* _
       }
       return;
     }
-    // [head][chunk][lpp lanes][m, s, o.xyzw] through to memory
-    u32* pp = reinterpret_cast<u32*>(partial) + ((static_cast<size_t>(head) * chunks + ci) * lpp + sub) * 8u;
-    const float vals[6] = {st.m, st.s, st.o.x, st.o.y, st.o.z, st.o.w};
-#pragma unroll
-    for (int i = 0; i < 6; ++i) __hip_atomic_store(pp + i, __float_as_uint(vals[i]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // [head][chunk][lpp lanes][m, s, -, -, o.xyzw] through to memory: two 16-byte stores at agent scope
+    const u32 slot = static_cast<u32>(((static_cast<size_t>(head) * chunks + ci) * lpp + sub) * 32u);
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(st.m), __float_as_uint(st.s), 0u, 0u}, part_rsrc, static_cast<int>(slot), 0, 16);
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(st.o.x), __float_as_uint(st.o.y), __float_as_uint(st.o.z), __float_as_uint(st.o.w)},
+                                           part_rsrc, static_cast<int>(slot + 16u), 0, 16);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (lane == 0u) {
       const u32 old = __hip_atomic_fetch_add(counters + head, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -110,18 +113,21 @@ __device__ __forceinline__ void body(const float* __restrict__ q, const float* _
   __syncthreads();
   if (wave != 0u || lane >= lpp || s_old != chunks - 1u) return;
   State tot = {-INFINITY, 0.0f, zero4};
-  for (u32 c0 = 0; c0 < chunks; c0 += 8u) {        // eight chunks' states in flight, merged in chunk order
-    float vals[8][6];
+  constexpr u32 kRound = 16;                       // chunks whose states are in flight together; merged in chunk order
+  for (u32 c0 = 0; c0 < chunks; c0 += kRound) {
+    u32x4 ms[kRound], ov[kRound];
 #pragma unroll
-    for (u32 cc = 0; cc < 8; ++cc) {
+    for (u32 cc = 0; cc < kRound; ++cc) {
       const u32 c = min(c0 + cc, chunks - 1u);
-      const u32* pp = reinterpret_cast<const u32*>(partial) + ((static_cast<size_t>(head) * chunks + c) * lpp + sub) * 8u;
-#pragma unroll
-      for (int i = 0; i < 6; ++i) vals[cc][i] = __uint_as_float(__hip_atomic_load(pp + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      const u32 slot = static_cast<u32>(((static_cast<size_t>(head) * chunks + c) * lpp + sub) * 32u);
+      ms[cc] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, static_cast<int>(slot), 0, 16);
+      ov[cc] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, static_cast<int>(slot + 16u), 0, 16);
     }
 #pragma unroll
-    for (u32 cc = 0; cc < 8; ++cc)
-      if (c0 + cc < chunks) merge(tot, vals[cc][0], vals[cc][1], f32x4{vals[cc][2], vals[cc][3], vals[cc][4], vals[cc][5]});
+    for (u32 cc = 0; cc < kRound; ++cc)
+      if (c0 + cc < chunks)
+        merge(tot, __uint_as_float(ms[cc].x), __uint_as_float(ms[cc].y),
+              f32x4{__uint_as_float(ov[cc].x), __uint_as_float(ov[cc].y), __uint_as_float(ov[cc].z), __uint_as_float(ov[cc].w)});
   }
   if (live) {
     const float inv = 1.0f / tot.s;

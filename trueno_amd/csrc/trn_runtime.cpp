@@ -82,6 +82,7 @@ int g_tune_stream_consumers = 0;
 int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
 int g_tune_gemm_ksplit = 0;     // parts of K in the matrix-core GEMM (0: chosen from the shape)
+int g_tune_attention_per_cu = 0;   // workgroups per CU the single-query attention aims at (0: default)
 int g_tune_gemm_waves = 0;      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
@@ -302,7 +303,8 @@ hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t
   while ((4u << lpp_log2) < head_dim) ++lpp_log2;
   const uint32_t lpp = 1u << lpp_log2, step = 4u * (64u >> lpp_log2);       // positions a workgroup takes at a time
   // chunks of positions per head: about two workgroups per CU, at least four steps each
-  uint32_t chunks = std::max(1u, (2u * uint32_t(d->cu_count) + num_heads - 1u) / num_heads);
+  const uint32_t per_cu = g_tune_attention_per_cu > 0 ? uint32_t(g_tune_attention_per_cu) : 2u;
+  uint32_t chunks = std::max(1u, (per_cu * uint32_t(d->cu_count) + num_heads - 1u) / num_heads);
   chunks = std::max(1u, std::min(chunks, (seq_len + 4u * step - 1u) / (4u * step)));
   uint32_t chunk = (seq_len + chunks - 1u) / chunks;
   chunk = (chunk + step - 1u) / step * step;
@@ -1298,6 +1300,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "attention_per_cu")) { g_tune_attention_per_cu = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
