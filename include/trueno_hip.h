@@ -238,7 +238,9 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
  * "group_off": 1 = in mode 0 never fuse neighbouring independent entries of a list into one launch.
  * "gemm_mfma_off": 1 = the Q4_K GEMM never takes the matrix-core form; "gemm_k_parts": into how many parts
- * that form cuts K (0 = chosen from the shape); "gemm_waves": 4 or 8 strips of 32 rows per workgroup (0 = 8). */
+ * that form cuts K (0 = chosen from the shape); "gemm_waves": 4 or 8 strips of 32 rows per workgroup (0 = 8);
+ * "attention_per_cu": workgroups per CU the single-query attention aims at (0 = 2); "attention_min_steps": least
+ * number of steps (of 8 positions at head_dim 128) in a chunk of positions (0 = 8). */
 TRN_API trn_status trn_set_tuning(const char* key, int value);
 
 #ifdef __cplusplus
