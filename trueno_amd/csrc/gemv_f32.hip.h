@@ -27,6 +27,8 @@ __device__ __forceinline__ void fast_body(float* __restrict__ y, const float* __
   const u32 k0 = part * rows_per_part, k1 = min(k_dim, k0 + rows_per_part);
   const f32x4* ap = reinterpret_cast<const f32x4*>(a + (col_ok ? col : 0u));
   const size_t stride4 = n_dim >> 2;
+  const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      partial, 0, static_cast<int>(min(static_cast<size_t>(0x7FFFFFFF), static_cast<size_t>(parts) * n_dim * 4u)), 0x00020000);
   f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
   u32 k = k0 + wave;
   for (; k + (kUnroll - 1u) * kWaves < k1; k += kUnroll * kWaves) {
@@ -61,13 +63,9 @@ __device__ __forceinline__ void fast_body(float* __restrict__ y, const float* __
       if (col_ok) *reinterpret_cast<f32x4*>(y + col) = acc;
       return;
     }
-    if (col_ok) {
-      u32* dst = reinterpret_cast<u32*>(partial + static_cast<size_t>(part) * n_dim + col);
-      __hip_atomic_store(dst + 0, __float_as_uint(acc.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(dst + 1, __float_as_uint(acc.y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(dst + 2, __float_as_uint(acc.z), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(dst + 3, __float_as_uint(acc.w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (col_ok)      // across workgroups (and XCDs): one 16-byte buffer store at agent scope (sc1)
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(acc.x), __float_as_uint(acc.y), __float_as_uint(acc.z), __float_as_uint(acc.w)},
+                                             part_rsrc, static_cast<int>((part * n_dim + col) * 4u), 0, 16);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the coherent stores have been acknowledged
     if (lane == 0u) {
       const u32 old = __hip_atomic_fetch_add(counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -78,21 +76,17 @@ __device__ __forceinline__ void fast_body(float* __restrict__ y, const float* __
   __syncthreads();
   if (wave != 0u || s_old != parts - 1u || !col_ok) return;
   float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (u32 p0 = 0; p0 < parts; p0 += 8u) {                 // up to 32 loads in flight, added in part order
-    u32 got[8][4];
+  for (u32 p0 = 0; p0 < parts; p0 += 16u) {                // sixteen parts in flight, added in part order
+    u32x4 got[16];
 #pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp)
+    for (u32 pp = 0; pp < 16; ++pp)
+      got[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, static_cast<int>((min(p0 + pp, parts - 1u) * n_dim + col) * 4u), 0, 16);
 #pragma unroll
-      for (u32 i = 0; i < 4; ++i) {
-        got[pp][i] = 0u;
-        if (p0 + pp < parts)
-          got[pp][i] = __hip_atomic_load(reinterpret_cast<const u32*>(partial + static_cast<size_t>(p0 + pp) * n_dim + col) + i,
-                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (u32 pp = 0; pp < 16; ++pp)
+      if (p0 + pp < parts) {
+        r[0] += __uint_as_float(got[pp].x); r[1] += __uint_as_float(got[pp].y);
+        r[2] += __uint_as_float(got[pp].z); r[3] += __uint_as_float(got[pp].w);
       }
-#pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp)
-#pragma unroll
-      for (u32 i = 0; i < 4; ++i) r[i] += __uint_as_float(got[pp][i]);
   }
   *reinterpret_cast<f32x4*>(y + col) = f32x4{r[0], r[1], r[2], r[3]};
 }

@@ -355,17 +355,19 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
       }
     return;
   }
-  // several parts of K: publish this part, the last arrival adds them up
-  if (row_ok)
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
-        if (token < m)
-          __hip_atomic_store(reinterpret_cast<u32*>(partial) + (static_cast<size_t>(part) * tokens_pad + token) * n + row,
-                             __float_as_uint(val[2 * a + b]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+  // several parts of K: publish this part, the last arrival adds them up.  The parts cross workgroups (and XCDs):
+  // 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side by side:
+  //   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
+  const u32 strips = groups * waves;
+  const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      partial, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
+  auto slot_of = [&](u32 pt) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
+  __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[0]), __float_as_uint(val[1]), __float_as_uint(val[2]), __float_as_uint(val[3])},
+                                         part_rsrc, slot_of(part), 0, 16);
+  const bool upper = tile * kTokensPerTile + 8u < m;      // tokens 8..15 of the tile exist (val[4..7])
+  if (upper)
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[4]), __float_as_uint(val[5]), __float_as_uint(val[6]), __float_as_uint(val[7])},
+                                           part_rsrc, slot_of(part) + 16, 0, 16);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
   asm volatile("s_barrier" ::: "memory");
   if (threadIdx.x == 0u) {
@@ -379,22 +381,20 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
     __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (old != kparts - 1u || !row_ok) return;
   float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // up to 64 loads in flight, added in part order
-    u32 got[8][8];
+  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // eight parts in flight, added in part order
+    u32x4 lo[8], hi[8];
 #pragma unroll
-    for (int pp = 0; pp < 8; ++pp)
+    for (u32 pp = 0; pp < 8; ++pp) {
+      const u32 pt = min(p0 + pp, kparts - 1u);
+      lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
+      hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
-        got[pp][t] = 0u;
-        if (p0 + pp < kparts && token < m)
-          got[pp][t] = __hip_atomic_load(reinterpret_cast<const u32*>(partial) + (static_cast<size_t>(p0 + pp) * tokens_pad + token) * n + row,
-                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (u32 pp = 0; pp < 8; ++pp)
+      if (p0 + pp < kparts) {
+        r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
+        r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
       }
-#pragma unroll
-    for (int pp = 0; pp < 8; ++pp)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) r[t] += __uint_as_float(got[pp][t]);
   }
 #pragma unroll
   for (int t = 0; t < 8; ++t) {

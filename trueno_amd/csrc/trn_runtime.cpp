@@ -362,7 +362,8 @@ hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a,
   kparts = (nsb + ksb - 1u) / ksb;
   auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
   const size_t cnt_bytes = up(size_t(groups) * tiles * 4u);
-  const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * 16u * n * 4u) : 0u;
+  // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
+  const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * groups * waves * 2048u) : 0u;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
