@@ -8,6 +8,9 @@
 // 32-thread warp, :1151-1155): here it is a property of the kernel, chosen by the host library,
 // and every kernel gives the same result for any grid size and any block size that is a
 // multiple of 64.
+#ifndef KQ_U
+#define KQ_U 2      // rows a wave of the fast GEMV engine has in flight (the host's kGemvRowsPerBatch)
+#endif
 #include "kquant_chain.hip.h"
 #include "kquant_stream.hip.h"
 #include "kquant_gemm_f16.hip.h"
@@ -67,14 +70,14 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, 0u, w, x, y};                                               \
-    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
+    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(768)                                                      \
       fmtname##_gemv_flags(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) {\
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
-    chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
+    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
@@ -100,15 +103,15 @@ extern "C" __global__ void __launch_bounds__(768) kq_gemv_group(const GemvGroup 
   while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) ++i;
   const ChainEntry e = g.e[i];
   const u32 block_id = blockIdx.x - g.first[i], num_blocks = g.first[i + 1] - g.first[i];
-  if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
-  else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
-  else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
+  if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
+  else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
+  else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
 }
 
 // The list as phases of independent entries in one resident launch, one workgroup of 12 waves per CU.
 extern "C" __global__ void __launch_bounds__(768)
 kq_gemv_phases(const ChainEntry* entries, const PhaseAssign* assign, u32 phases, u32* counters, u32* status, u32 spin_limit) {
-  phases_body<2>(entries, assign, phases, counters, status, spin_limit);
+  phases_body<KQ_U>(entries, assign, phases, counters, status, spin_limit);
 }
 
 // The list with decoupled weight streaming (kquant_stream.hip.h): one workgroup per CU.
@@ -226,7 +229,7 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
     for (u32 r = blockIdx.y; r < m; r += gridDim.y) {                                                    \
       const ChainEntry e = {FMT, k, n, 0u, b_quant, a + static_cast<size_t>(r) * k,                      \
                             c + static_cast<size_t>(r) * n};                                             \
-      chain_step<FMT, 2>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                        \
+      chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                        \
       __syncthreads();                                                                                   \
     }                                                                                                    \
   }                                                                                                      \

@@ -47,7 +47,10 @@ enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED =
             KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8, KIND_ATTENTION = 9 };
 
 constexpr int kMaxDevices = 64;
-constexpr uint32_t kGemvRowsPerBatch = 2;     // U of the fast GEMV kernel
+#ifndef KQ_U
+#define KQ_U 2
+#endif
+constexpr uint32_t kGemvRowsPerBatch = KQ_U;  // U of the fast GEMV kernel (the build passes it to both sides)
 constexpr uint32_t kGemvMaxWaves = 12;        // __launch_bounds__(768) of the fast GEMV kernels
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
