@@ -86,6 +86,7 @@ int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
 int g_tune_gemm_ksplit = 0;     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 int g_tune_attention_min_steps = 0;
+int g_tune_slab_weight = 0;        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 int g_tune_attention_per_cu = 0;   // workgroups per CU the single-query attention aims at (0: default)
 int g_tune_gemm_waves = 0;      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
 
@@ -1117,8 +1118,17 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     const GemvGeometry alone = gemv_geometry(*d, descs[i].k, descs[i].n);
     if (!alone.fits) return hipErrorInvalidValue;
     waves = std::max(waves, alone.block / 64u);
-    total_bytes += double(descs[i].n) * (descs[i].k / 256u) * kSbBytes[descs[i].fmt - 4];
   }
+  // What an entry costs a workgroup is not only its bytes: with k > 4096 every workgroup stages a larger vector and
+  // the waves that share a row meet in LDS.  Measured on [Q6_K 4096x11008 + 3 x Q4_K 4096x4096]: with shares by bytes
+  // the wide entry's workgroups end 5 us after the others; counting its bytes 1.6-1.75 times is best (0.3 per
+  // further slab of 4096 columns; "group_slab_weight" overrides the percentage).
+  auto cost_of = [&](const trn_gemv_desc& e) {
+    const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
+    const double per_slab = (g_tune_slab_weight > 0 ? g_tune_slab_weight : 30) / 100.0;
+    return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
+  };
+  for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
   // the kernels hold 3 waves per SIMD, 12 per CU
   const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::max(1u, 12u / waves);
   const double target = double(d->cu_count) * per_cu;
@@ -1128,8 +1138,10 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   for (uint32_t i = 0; i < len; ++i) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves), groups = waves / sw;
-    const uint32_t ug = kGemvRowsPerBatch * groups;
-    const double bytes = double(e.n) * nsb * kSbBytes[e.fmt - 4];
+    // workgroups of 8 waves or more hand their row batches out among the waves: a share need not be a whole
+    // number of rounds of all waves
+    const uint32_t ug = waves >= 8u ? kGemvRowsPerBatch : kGemvRowsPerBatch * groups;
+    const double bytes = cost_of(e);
     const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
     uint64_t rows = (uint64_t(e.n) + share - 1) / share;
     rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
@@ -1307,6 +1319,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_slab_weight")) { g_tune_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_per_cu")) { g_tune_attention_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_min_steps")) { g_tune_attention_min_steps = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
