@@ -430,7 +430,7 @@ def main() -> int:
         layer_bytes = sum(alg_bytes(fmt, n, k) for _, fmt, n, k in LAYER_MATS)
         reps, spent = 0, 0.0
         t_start = time.time()
-        while (spent < 10.0 and reps < 200) or reps < 2:
+        while (spent < 10.0 and reps < 4000) or reps < 2:      # about 10 s of wall time on all the job's cores
             for name, fmt, n, k in LAYER_MATS:
                 _, sec = cb.dequant_matvec(fmt, host_layer0[name], hx[k], k, n, cores, 1)
                 spent += sec
