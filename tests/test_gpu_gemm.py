@@ -138,3 +138,20 @@ def test_q4k_gemm_special_values(gpu):
     for i in (0, 2, 3):
         assert kq.rel_l2(c[i], c64[i]) <= TOL
     assert not np.any(np.isfinite(c[4]))
+
+
+def test_gemm_on_streams_that_come_and_go(gpu):
+    """the scratch buffers a stream's products use (partial sums, arrival counters) go with the stream; a new stream,
+    possibly with the old one's handle, starts from clean ones"""
+    ctx, _ = gpu
+    n, k, m = 1024, 4096, 4                       # K is cut in parts on this shape: partial sums and counters in use
+    buf, a = kq.gen_matrix("q4k", 91, n, k), kq.gen_x(92, m, k)
+    want = _c64("q4k", buf, a, n, k)
+    first = None
+    for _ in range(3):
+        stream = t.CudaStream(ctx)
+        c = gpu_gemm((ctx, stream), "q4k", buf, a, m, n, k)
+        assert kq.rel_l2(c, want) <= TOL
+        first = c if first is None else first
+        assert np.array_equal(c.view(np.uint32), first.view(np.uint32))
+        stream.destroy()

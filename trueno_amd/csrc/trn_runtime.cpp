@@ -991,9 +991,45 @@ trn_status trn_stream_create(trn_stream* stream, unsigned flags) {
   return TRN_SUCCESS;
 }
 
+// The per-(device, stream) scratch buffers of a stream that is going away (partial sums, arrival counters, the
+// resident executor's tables).  The stream must be idle.
+static void release_stream_workspaces(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto drop_simple = [&](auto& map) {
+    for (auto it = map.begin(); it != map.end();) {
+      if (it->first.second == stream) {
+        if (it->second.buf) (void)hipFree(it->second.buf);
+        it = map.erase(it);
+      } else {
+        ++it;
+      }
+    }
+  };
+  drop_simple(g_gemv_f32_ws);
+  drop_simple(g_attention_ws);
+  drop_simple(g_gemm_ws);
+  for (auto it = g_chain_ws.begin(); it != g_chain_ws.end();) {
+    if (it->first.second == stream) {
+      ChainWorkspace& w = it->second;
+      if (w.d_entries) (void)hipFree(w.d_entries);
+      if (w.d_counters) (void)hipFree(w.d_counters);
+      if (w.d_assign) (void)hipFree(w.d_assign);
+      if (w.h_status) (void)hipHostFree(w.h_status);
+      it = g_chain_ws.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+
 trn_status trn_stream_destroy(trn_stream stream) {
   if (!stream) return TRN_ERROR_INVALID_VALUE;
-  return st(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // work that still uses the stream's scratch buffers must have finished before they are freed
+  const hipError_t e = hipStreamSynchronize(s);
+  release_stream_workspaces(s);
+  const hipError_t d = hipStreamDestroy(s);
+  return st(e != hipSuccess ? e : d);
 }
 
 trn_status trn_stream_synchronize(trn_stream stream) { return st(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
