@@ -183,30 +183,30 @@ def main() -> int:
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
     assert np.all(np.isfinite(logits.copy_to_host())), "the pass produced non-finite logits"
 
-    # ---- dominant kernel: kq_gemv_group.  The library fuses neighbouring independent entries (up to four) into one
-    #      launch of this kernel: [q,k,v] of the first layer, then per layer [o,gate,up] and [down, q',k',v' of the
-    #      next layer] - 64 launches that carry all of the pass but the last down and the head (3.99 of 4.13 GB).
-    #      Those 64 launches, in pass order, back to back on the stream, bracketed by HIP events on that stream.
-    entries = []
-    for layer in range(layers):
-        for name, fmt, n, k in LAYER_MATS:
-            src = src_of[name]
-            x, flags = (xs[layer][0], 0) if src is None else (act[src], NORM)
-            entries.append((fmt, k, n, act[name], weights[layer][name], x, flags))
-    cuts = [(0, 3)]
-    for layer in range(layers):
-        base = 7 * layer
-        cuts.append((base + 3, base + 6))
-        if layer + 1 < layers:
-            cuts.append((base + 6, base + 10))
+    # ---- dominant kernel: kq_gemv_group.  The library puts entries that are independent of one another (and of what
+    #      they would overtake) into one launch of this kernel; trn_kquant_gemv_plan says which entry of the pass goes
+    #      into which launch.  The launches of the pass that hold two or more entries (all of it but a few single
+    #      GEMVs, which take the single-GEMV kernels) are issued here one list each, in pass order, back to back on
+    #      the stream, bracketed by HIP events on that stream.
+    launch_of = batch.plan()
+    members = {}
+    for i, l in enumerate(launch_of):
+        members.setdefault(l, []).append(i)
+    entry_bytes = [alg_bytes(fmt, n, k) for _ in range(layers) for _, fmt, n, k in LAYER_MATS] + [alg_bytes(HEAD[1], HEAD[2], HEAD[3])]
+    entry_names = [name for _ in range(layers) for name, _, _, _ in LAYER_MATS] + ["head"]
+    kinds = {}
+    for l in sorted(members):
+        sig = "[" + ",".join(entry_names[i] for i in members[l]) + "]"
+        kinds[sig] = kinds.get(sig, 0) + 1
+    print("[bench] launches of the pass: " + ", ".join(f"{c} x {sig}" for sig, c in kinds.items()), file=sys.stderr, flush=True)
     groups = []
     grp_bytes = 0
-    for a, b in cuts:
-        g = t.GemvBatch()
-        for fmt, k, n, yb, wb, xb, flags in entries[a:b]:
-            g.add(fmt, k, n, yb, wb, xb, flags)
-            grp_bytes += alg_bytes(fmt, n, k)
-        groups.append(g)
+    for l in sorted(members):
+        if len(members[l]) >= 2:
+            g = batch.subset(members[l])
+            assert len(set(g.plan())) == 1, "a launch of the pass, issued alone, must again be one launch"
+            groups.append(g)
+            grp_bytes += sum(entry_bytes[i] for i in members[l])
     n_grp = len(groups)
     e0, e1 = ev(), ev()
     grp_ms = []

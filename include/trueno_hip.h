@@ -130,14 +130,16 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * roadmap.yaml:359-368).  Entry i computes y = dequant(W) x exactly as the typed launcher of its
  * format would; a later entry may read what an earlier one wrote (the library finds those
  * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
- * By default the list is issued as one launch per entry, except that up to four neighbouring entries
- * that do not touch one another's vectors (q, k, v of a decoder layer; gate and up) share one launch.
+ * By default (mode 0) entries that do not touch one another's vectors share a launch, up to eight: the first
+ * entry still waiting, plus later ones of a window of the list (q, k, v of a decoder layer; gate and up; ...)
+ * that depend neither on it nor on anything they would overtake.  What an entry computes does not depend on the
+ * company it is launched in: the results are, bit for bit, those of one launch per entry in list order.
  * With trn_set_tuning("batch_mode", 1 or 2), and when every entry meets the fast kernels' alignment (x 16 B,
  * W 16 B / 2 B for Q6_K), the list runs as ONE cooperative launch of resident workgroups: the list is cut in
  * phases of mutually independent entries with a device-side barrier between phases (mode 1), or a producer wave
  * per CU streams the weights through an LDS ring (mode 2).  These forms keep, per (device, stream), small device
  * buffers with the list, the work assignment and the barrier counters (allocated on first use, kept until the
- * process ends); a list identical to the previous one on that stream is not uploaded again.  If a device-side
+ * stream is destroyed); a list identical to the previous one on that stream is not uploaded again.  If a device-side
  * wait ever runs out of its (seconds-long) spin budget the kernel exits and the next call on that stream returns
  * hipErrorLaunchFailure (719).  All three forms give bit-identical results. */
 /* An entry may fold the element-wise steps of a decoder layer in (zero pointers: absent):
@@ -165,6 +167,9 @@ typedef struct trn_gemv_desc {
   uint32_t reserved;   /* 0 */
 } trn_gemv_desc;
 TRN_API trn_status trn_kquant_gemv_batch(trn_stream stream, const trn_gemv_desc* descs, uint32_t count);
+/* Which launch of mode 0 each entry of the list would go into: launch_of[i] = 0, 1, ... in launch order.  Launches
+ * nothing (for tools that want to time or describe the launches of a list; no counterpart in the reference). */
+TRN_API trn_status trn_kquant_gemv_plan(const trn_gemv_desc* descs, uint32_t count, uint32_t* launch_of);
 
 /* ---- 9. test surface: dequantise to f32 (no counterpart in the reference) ------------------------
  * out[sb*256 + i] = weight i of super-block sb.  policy 0 = GEMV-family decode
@@ -236,7 +241,9 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * barriers, 2 as 1 with a producer wave per CU streaming the weights through an LDS ring.
  * "stream_consumers": consumer waves of mode 2.
  * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
- * "group_off": 1 = in mode 0 never fuse neighbouring independent entries of a list into one launch.
+ * "group_off": 1 = in mode 0 one launch per entry; "group_max": most entries in a launch (0 = 8); "group_window":
+ * how far down the list a launch looks for entries (0 = 16); "group_slab_weight": percent added to an entry's
+ * bytes per further 4096 columns when a launch shares out its workgroups (0 = 30).
  * "gemm_mfma_off": 1 = the Q4_K GEMM never takes the matrix-core form; "gemm_k_parts": into how many parts
  * that form cuts K (0 = chosen from the shape); "gemm_waves": 4 or 8 strips of 32 rows per workgroup (0 = 8);
  * "attention_per_cu": workgroups per CU the single-query attention aims at (0 = 2); "attention_min_steps": least

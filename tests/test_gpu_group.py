@@ -74,3 +74,38 @@ def test_grouped_equals_separate(gpu, case):
         if flags:
             ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
         assert kq.rel_l2(got[dst], ref) <= TOL, (case, dst)
+
+
+@pytest.mark.parametrize("seed", (0, 1, 2, 3))
+def test_entries_brought_forward_keep_the_lists_meaning(gpu, seed):
+    """A launch may take entries from further down the list when nothing they touch is touched by an entry they
+    overtake.  Random lists over a small pool of vectors (so that read-after-write, write-after-read and
+    write-after-write all occur, also in place) must leave every vector with the bits of one launch per entry."""
+    rng = np.random.default_rng(seed)
+    dim = 512
+    names = [f"v{i}" for i in range(6)]
+    specs = []
+    for i in range(20):
+        src, dst = rng.choice(names, 2, replace=False)
+        specs.append((("q4k", "q5k", "q6k")[int(rng.integers(3))], dim, dim, str(src), str(dst), 1))
+
+    def run(group_off):
+        ctx, stream = gpu
+        bufs = {nm: t.GpuBuffer.from_host(ctx, kq.gen_x(50 + j, dim)) for j, nm in enumerate(names)}
+        keep, batch = [], t.GemvBatch()
+        for i, (fmt, n, k, src, dst, flags) in enumerate(specs):
+            w = t.GpuBuffer.from_host(ctx, kq.gen_matrix(fmt, 7000 + 100 * seed + i, n, k))
+            keep.append(w)
+            batch.add(fmt, k, n, bufs[dst], w, bufs[src], flags)
+        _tune("group_off", group_off)
+        try:
+            batch.launch(stream)
+            stream.synchronize()
+        finally:
+            _tune("group_off", 0)
+        return {nm: b.copy_to_host() for nm, b in bufs.items()}
+
+    want, got = run(1), run(0)
+    for nm in names:
+        assert np.all(np.isfinite(want[nm])), nm
+        assert np.array_equal(want[nm].view(np.uint32), got[nm].view(np.uint32)), (seed, nm)

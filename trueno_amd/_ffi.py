@@ -57,6 +57,7 @@ SIGNATURES = {
     "trn_rmsnorm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_float],
     "trn_fused_residual_rmsnorm": [vp, dptr, dptr, dptr, dptr, C.c_uint32, C.c_float],
     "trn_kquant_gemv_batch": [vp, vp, C.c_uint32],
+    "trn_kquant_gemv_plan": [vp, C.c_uint32, vp],
     "trn_q4k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q5k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],
     "trn_q6k_dequant_f32": [vp, dptr, dptr, C.c_uint64, C.c_int],

@@ -88,12 +88,12 @@ KQ_GEMV_KERNELS(q4k, FMT_Q4K)
 KQ_GEMV_KERNELS(q5k, FMT_Q5K)
 KQ_GEMV_KERNELS(q6k, FMT_Q6K)
 
-// Up to four GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
+// Up to eight GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
 // up) in one launch: consecutive runs of workgroups belong to consecutive entries.  Each entry is computed
 // exactly as its own launch would compute it.
 struct GemvGroup {
-  ChainEntry e[4];
-  u32 first[5];      // first[i] .. first[i+1]-1 are the workgroups of entry i
+  ChainEntry e[8];
+  u32 first[9];      // first[i] .. first[i+1]-1 are the workgroups of entry i
   u32 count;
 };
 extern "C" __global__ void __launch_bounds__(768) kq_gemv_group(const GemvGroup g) {

@@ -86,6 +86,8 @@ int g_tune_group_off = 0;
 int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
 int g_tune_gemm_ksplit = 0;     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 int g_tune_attention_min_steps = 0;
+int g_tune_group_window = 0;       // entries of a list a grouped launch may look ahead over (0: 16)
+int g_tune_group_max = 0;          // most entries in one grouped launch (0: 8)
 int g_tune_slab_weight = 0;        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 int g_tune_attention_per_cu = 0;   // workgroups per CU the single-query attention aims at (0: default)
 int g_tune_gemm_waves = 0;      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
@@ -1134,16 +1136,17 @@ trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
 }
 
 namespace {
+constexpr uint32_t kGroupMax = 8;      // entries of one grouped launch
 struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip
-  ChainEntryHost e[4];
-  uint32_t first[5];
+  ChainEntryHost e[kGroupMax];
+  uint32_t first[kGroupMax + 1];
   uint32_t count;
 };
-static_assert(sizeof(GemvGroupHost) == 4 * 72 + 5 * 4 + 4, "GemvGroup layout");
+static_assert(sizeof(GemvGroupHost) == kGroupMax * 72 + (kGroupMax + 1) * 4 + 4, "GemvGroup layout");
 
 bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
-// Entries first .. first+len-1 of a list (len in 2..4, mutually independent, all meeting the fast kernels'
+// Entries first .. first+len-1 of an array (len in 1..kGroupMax, mutually independent, all meeting the fast kernels'
 // preconditions) as ONE launch.  The workgroups are as large as the largest entry needs (k > 4096 wants one
 // wave per slab of 4096 columns), every entry gets a share of the resident workgroups in proportion to its
 // bytes, and an entry's rows are cut evenly over its share.
@@ -1234,6 +1237,56 @@ trn_status trn_fused_residual_rmsnorm(trn_stream s, trn_dptr residual, trn_dptr 
   return st(launch_rmsnorm(static_cast<hipStream_t>(s), residual, input, output, gamma, hidden_size, epsilon, true));
 }
 
+namespace {
+bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
+  return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
+         gemv_geometry(*dk, d.k, d.n).fits;
+}
+
+// Cuts a list into launches (mode 0).  A launch is filled with up to kGroupMax entries that are independent of one
+// another AND of every earlier entry that has not been launched yet: the first entry still waiting always goes in,
+// later ones of a window are brought forward when nothing they read or write is touched by an entry they would
+// overtake.  What an entry computes does not depend on the company it is launched in, so the results are those of
+// the list in order.
+void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches) {
+  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 16u);
+  const uint32_t group_max =
+      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupMax);
+  std::vector<uint8_t> launched(count, 0);
+  for (uint32_t pos = 0; pos < count;) {
+    if (launched[pos]) { ++pos; continue; }
+    std::vector<uint32_t> members(1, pos);
+    if (list_groupable(dk, descs[pos])) {
+      const uint32_t end = uint32_t(std::min<uint64_t>(count, uint64_t(pos) + window));
+      for (uint32_t j = pos + 1; j < end && members.size() < group_max; ++j) {
+        if (launched[j]) continue;
+        const trn_gemv_desc& c = descs[j];
+        if (!list_groupable(dk, c)) break;           // an entry that takes another path keeps its place in the order
+        bool ok = true;
+        for (uint32_t i = pos; i < j && ok; ++i)     // the members of the launch and everything it would overtake
+          if (!launched[i]) ok = !gemv_depends(c, descs[i]) && !gemv_depends(descs[i], c);
+        if (ok) members.push_back(j);
+      }
+    }
+    for (uint32_t m : members) launched[m] = 1;
+    launches->push_back(std::move(members));
+  }
+}
+}  // namespace
+
+trn_status trn_kquant_gemv_plan(const trn_gemv_desc* descs, uint32_t count, uint32_t* launch_of) {
+  if (count == 0) return TRN_SUCCESS;
+  if (!descs || !launch_of) return TRN_ERROR_INVALID_VALUE;
+  DeviceKernels* dk = nullptr;
+  hipError_t e = device_kernels(&dk);
+  if (e != hipSuccess) return st(e);
+  std::vector<std::vector<uint32_t>> launches;
+  schedule_list(dk, descs, count, &launches);
+  for (size_t l = 0; l < launches.size(); ++l)
+    for (uint32_t m : launches[l]) launch_of[m] = uint32_t(l);
+  return TRN_SUCCESS;
+}
+
 trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {
   if (count == 0) return TRN_SUCCESS;
   if (!descs) return TRN_ERROR_INVALID_VALUE;
@@ -1248,33 +1301,22 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   if (handled || e != hipSuccess) return st(e);
   DeviceKernels* dk = nullptr;
   if ((e = device_kernels(&dk)) != hipSuccess) return st(e);
-  auto groupable = [&](const trn_gemv_desc& d) {
-    return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
-           gemv_geometry(*dk, d.k, d.n).fits;
-  };
-  for (uint32_t i = 0; i < count;) {
-    // longest run (up to 4) of entries that do not touch one another's vectors
-    uint32_t len = 1;
-    if (!g_tune_group_off && groupable(descs[i])) {
-      while (len < 4 && i + len < count) {
-        const trn_gemv_desc& c = descs[i + len];
-        bool ok = groupable(c);
-        for (uint32_t j = i; j < i + len && ok; ++j) ok = !gemv_depends(c, descs[j]) && !gemv_depends(descs[j], c);
-        if (!ok) break;
-        ++len;
-      }
-    }
-    if (len >= 2 || (desc_extended(descs[i]) && groupable(descs[i]))) {
-      e = launch_gemv_group(dk, stream, descs + i, len);
-    } else if (desc_extended(descs[i])) {
+  std::vector<std::vector<uint32_t>> launches;
+  schedule_list(dk, descs, count, &launches);
+  std::vector<trn_gemv_desc> group;
+  for (const std::vector<uint32_t>& members : launches) {
+    const trn_gemv_desc& head = descs[members[0]];
+    if (members.size() >= 2 || (desc_extended(head) && list_groupable(dk, head))) {
+      group.clear();
+      for (uint32_t m : members) group.push_back(descs[m]);
+      e = launch_gemv_group(dk, stream, group.data(), uint32_t(group.size()));
+    } else if (desc_extended(head)) {
       // folded element-wise steps need the fast engine (x, x2, gamma 16-byte aligned; the vector and a row block in LDS)
       return TRN_ERROR_INVALID_VALUE;
     } else {
-      const trn_gemv_desc& d = descs[i];
-      e = launch_gemm_like(Fmt(d.fmt - 4), stream, d.x, d.w, d.y, 1, d.n, d.k, true, d.flags);
+      e = launch_gemm_like(Fmt(head.fmt - 4), stream, head.x, head.w, head.y, 1, head.n, head.k, true, head.flags);
     }
     if (e != hipSuccess) return st(e);
-    i += len;
   }
   return TRN_SUCCESS;
 }
@@ -1355,6 +1397,8 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_window")) { g_tune_group_window = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_max")) { g_tune_group_max = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_slab_weight")) { g_tune_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_per_cu")) { g_tune_attention_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_min_steps")) { g_tune_attention_min_steps = value; return TRN_SUCCESS; }

@@ -237,6 +237,22 @@ class GemvBatch:
     def __len__(self) -> int:
         return len(self._entries)
 
+    def plan(self):
+        """launch_of[i]: which launch (0, 1, ... in launch order) the library's default mode puts entry i into.
+        Launches nothing."""
+        import ctypes as C
+        if self._array is None:
+            self._array = (_ffi.GemvDesc * len(self._entries))(*self._entries)
+        out = (C.c_uint32 * len(self._entries))()
+        _check(_lib().trn_kquant_gemv_plan(self._array, len(self._entries), out), "KernelLaunch", "kquant_gemv_plan")
+        return list(out)
+
+    def subset(self, indices) -> "GemvBatch":
+        """A list of the given entries of this one, in the given order."""
+        b = GemvBatch()
+        b._entries = [self._entries[i] for i in indices]
+        return b
+
     def launch(self, stream: CudaStream) -> None:
         if self._array is None:
             self._array = (_ffi.GemvDesc * len(self._entries))(*self._entries)
