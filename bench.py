@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the counter reads for kq_copy_u128 on
 # 256 MiB (profiles/kquant_gemv_hbm_traffic_pmc.md).  Counters cannot be read from inside this
 # process, so the figure is carried here and re-measured whenever the kernel changes.
-GROUP_TRAFFIC_BYTES_PER_LAUNCH = 62_891_367
+GROUP_TRAFFIC_BYTES_PER_LAUNCH = 63_595_450
 LAYERS = 32
 SB = {"q4k": 144, "q5k": 176, "q6k": 210}
 LAYER_MATS = [("q", "q4k", 4096, 4096), ("k", "q4k", 4096, 4096), ("v", "q4k", 4096, 4096), ("o", "q4k", 4096, 4096),
