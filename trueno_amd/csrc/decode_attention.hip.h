@@ -26,13 +26,34 @@ struct State {          // running softmax over some positions, in the 2^x domai
 };
 
 __device__ __forceinline__ void merge(State& a, float m, float s, const f32x4& o) {
-  const float nm = fmaxf(a.m, m);
-  const float ca = a.m == nm ? 1.0f : __builtin_amdgcn_exp2f(a.m - nm);     // -inf - -inf never reaches exp2
-  const float cb = m == nm ? 1.0f : __builtin_amdgcn_exp2f(m - nm);
+  // one of the two factors is always 1: a single exponential, of (smaller maximum - larger maximum)
+  const bool keep = a.m >= m;
+  const float nm = keep ? a.m : m, other = keep ? m : a.m;
+  const float e = other == nm ? 1.0f : __builtin_amdgcn_exp2f(other - nm);  // -inf - -inf never reaches exp2
+  const float ca = keep ? 1.0f : e, cb = keep ? e : 1.0f;
   a.s = a.s * ca + s * cb;
   a.o.x = a.o.x * ca + o.x * cb; a.o.y = a.o.y * ca + o.y * cb;
   a.o.z = a.o.z * ca + o.z * cb; a.o.w = a.o.w * ca + o.w * cb;
   a.m = nm;
+}
+
+// Sum of v over each group of 2^lpp_log2 neighbouring lanes, in every lane of the group, without going through LDS
+// (five dependent ds_bpermute per position cost more than the position's memory traffic): DPP within a row of 16
+// lanes, row sums through SGPRs beyond that.
+__device__ __forceinline__ float group_sum(float v, u32 lpp_log2, u32 lane) {
+  if (lpp_log2 >= 1u) v += dpp_f32<0xB1>(v);    // quad_perm [1,0,3,2]
+  if (lpp_log2 >= 2u) v += dpp_f32<0x4E>(v);    // quad_perm [2,3,0,1]
+  if (lpp_log2 >= 3u) v += dpp_f32<0x141>(v);   // row_half_mirror
+  if (lpp_log2 >= 4u) v += dpp_f32<0x140>(v);   // row_mirror: every lane of a row of 16 holds the row's sum
+  if (lpp_log2 >= 5u) {
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    const float lo = r0 + r1, hi = r2 + r3;
+    v = lpp_log2 >= 6u ? lo + hi : (lane < 32u ? lo : hi);
+  }
+  return v;
 }
 
 // lanes per position LPP = 2^lpp_log2 >= head_dim / 4
@@ -72,7 +93,7 @@ __device__ __forceinline__ void body(const float* __restrict__ q, const float* _
 #pragma unroll
     for (u32 a = 0; a < kAhead; ++a) {
       float d = fmaf(qv.w, kk[a].w, fmaf(qv.z, kk[a].z, fmaf(qv.y, kk[a].y, qv.x * kk[a].x)));
-      for (u32 off = 1; off < lpp; off <<= 1) d += __shfl_xor(d, off, 64);        // within the lane group
+      d = group_sum(d, lpp_log2, lane);
       if (p + a * stride < p1) merge(st, d * sl, 1.0f, vv[a]);
     }
   }
