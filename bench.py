@@ -447,6 +447,13 @@ def main() -> int:
                        "dequant_matvec_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_dq / 5) / 1e9, 2),
                        "matvec_predequantised_f32_us": round(sec_mv / 5 * 1e6, 1),
                        "matvec_predequantised_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_mv / 5) / 1e9, 2)}
+        # configurations 2 and 3 on the CPU path (dequantise + matvec per call)
+        for label, fmt, n, k in (("2_q6k_4096x4096", "q6k", 4096, 4096), ("2_q6k_32000x4096", "q6k", 32000, 4096),
+                                 ("3_q5k_11008x4096", "q5k", 11008, 4096), ("3_q5k_4096x11008", "q5k", 4096, 11008)):
+            wm = kq.gen_matrix(fmt, 1234 + n + k, n, k)
+            _, sec = cb.dequant_matvec(fmt, wm, hx[k], k, n, cores, 3)
+            cpu_config1[label] = {"dequant_matvec_us": round(sec / 3 * 1e6, 1),
+                                  "dequant_matvec_gbps_quantized": round(alg_bytes(fmt, n, k) / (sec / 3) / 1e9, 2)}
         cpu = {"value": round(layer_bytes * reps / spent / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"layer 0 of the pass (7 GEMVs, {layer_bytes / 1e6:.1f} MB quantized) x {reps} repetitions, "
                          f"dequantise-row + AVX2 dot, {'AVX2+FMA' if cb.has_avx2() else 'scalar'}"}
