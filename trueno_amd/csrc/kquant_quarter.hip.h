@@ -138,6 +138,8 @@ template <> struct Quarter<FMT_Q5K> {
     return (__umul24(bits4, 0x204081u) & 0x10101010u) | nibbles;
   }
 
+  // As for Q4_K the quants enter the FMAs as f16 subnormals: a 5-bit quant in the low bits of a 16-bit lane is
+  // q * 2^-24, and v_fma_mix_f32 takes it as it is; the factor leaves through the scale, every rounding unchanged.
   static __device__ __forceinline__ float dot(const Regs& r, u32 c, const float (&xr)[64], const float (&sx)[NSUM]) {
     float ds0, ds1, dm0, dm1;
     scales(r, ds0, ds1, dm0, dm1);
@@ -149,17 +151,19 @@ template <> struct Quarter<FMT_Q5K> {
       const u32 bh = t == 0 ? (r.qh.y << 4) & 0xF0u : (r.qh.y >> (4 * t - 4)) & 0xF0u;
       const u32 l = opaque(join5(v & 0x0F0F0F0Fu, bl));
       const u32 h = opaque(join5((v >> 4) & 0x0F0F0F0Fu, bh));
-      lo = fmaf(ubyte0(l), xr[4 * t + 0], lo);
-      lo = fmaf(ubyte1(l), xr[4 * t + 1], lo);
-      lo = fmaf(ubyte2(l), xr[4 * t + 2], lo);
-      lo = fmaf(ubyte3(l), xr[4 * t + 3], lo);
-      hi = fmaf(ubyte0(h), xr[32 + 4 * t + 0], hi);
-      hi = fmaf(ubyte1(h), xr[32 + 4 * t + 1], hi);
-      hi = fmaf(ubyte2(h), xr[32 + 4 * t + 2], hi);
-      hi = fmaf(ubyte3(h), xr[32 + 4 * t + 3], hi);
+      const h16x2 l02 = as_h16x2(l & 0x001F001Fu), l13 = as_h16x2((l >> 8) & 0x001F001Fu);   // bytes 0,2 and 1,3
+      const h16x2 h02 = as_h16x2(h & 0x001F001Fu), h13 = as_h16x2((h >> 8) & 0x001F001Fu);
+      lo = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], lo);
+      lo = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], lo);
+      lo = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], lo);
+      lo = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], lo);
+      hi = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], hi);
+      hi = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], hi);
+      hi = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], hi);
+      hi = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], hi);
     }
-    float acc = ds0 * lo;
-    acc = fmaf(ds1, hi, acc);
+    float acc = (ds0 * 16777216.0f) * lo;
+    acc = fmaf(ds1 * 16777216.0f, hi, acc);
     acc = fmaf(-dm0, sx[0], acc);
     acc = fmaf(-dm1, sx[1], acc);
     return acc;
