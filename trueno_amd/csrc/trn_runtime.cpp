@@ -518,27 +518,61 @@ std::map<std::pair<int, hipStream_t>, ChainWorkspace> g_chain_ws;
 uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u + (num_workgroups + 31u) / 32u); }
 
 
-bool desc_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
 // batch_mode 1: the list as phases of independent entries in ONE resident launch (kq_gemv_phases): one workgroup
 // of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
 // barrier between phases.  *handled = false (and hipSuccess): not possible here, issue the list the plain way.
-hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t stream, const trn_gemv_desc* descs,
-                         uint32_t count, bool* handled) {
-  constexpr uint32_t kWaves = kGemvMaxWaves, kMaxPerPhase = 16;
-  const uint32_t G = uint32_t(d->cu_count);
-  // phases: a new one starts where an entry touches a vector of an entry of the current phase
-  std::vector<std::pair<uint32_t, uint32_t>> ph;
-  uint32_t begin = 0;
-  for (uint32_t i = 0; i < count; ++i) {
-    bool dep = i - begin >= kMaxPerPhase || i - begin >= G;
-    for (uint32_t j = begin; j < i && !dep; ++j) dep = desc_depends(descs[i], descs[j]) || desc_depends(descs[j], descs[i]);
-    if (dep) {
-      ph.emplace_back(begin, i);
-      begin = i;
+constexpr uint32_t kGroupMax = 8;      // entries of one grouped launch
+bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
+  return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
+         gemv_geometry(*dk, d.k, d.n).fits;
+}
+
+// Cuts a list into launches (mode 0).  A launch is filled with up to kGroupMax entries that are independent of one
+// another AND of every earlier entry that has not been launched yet: the first entry still waiting always goes in,
+// later ones of a window are brought forward when nothing they read or write is touched by an entry they would
+// overtake.  What an entry computes does not depend on the company it is launched in, so the results are those of
+// the list in order.
+void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches) {
+  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 16u);
+  const uint32_t group_max =
+      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupMax);
+  std::vector<uint8_t> launched(count, 0);
+  for (uint32_t pos = 0; pos < count;) {
+    if (launched[pos]) { ++pos; continue; }
+    std::vector<uint32_t> members(1, pos);
+    if (list_groupable(dk, descs[pos])) {
+      const uint32_t end = uint32_t(std::min<uint64_t>(count, uint64_t(pos) + window));
+      for (uint32_t j = pos + 1; j < end && members.size() < group_max; ++j) {
+        if (launched[j]) continue;
+        const trn_gemv_desc& c = descs[j];
+        if (!list_groupable(dk, c)) break;           // an entry that takes another path keeps its place in the order
+        bool ok = true;
+        for (uint32_t i = pos; i < j && ok; ++i)     // the members of the launch and everything it would overtake
+          if (!launched[i]) ok = !desc_conflict(c, descs[i]) && !desc_conflict(descs[i], c);
+        if (ok) members.push_back(j);
+      }
     }
+    for (uint32_t m : members) launched[m] = 1;
+    launches->push_back(std::move(members));
   }
-  ph.emplace_back(begin, count);
+}
+
+hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t stream, const trn_gemv_desc* list,
+                         uint32_t count, bool* handled) {
+  constexpr uint32_t kWaves = kGemvMaxWaves;
+  const uint32_t G = uint32_t(d->cu_count);
+  // phases: the launches the list would be cut into (entries that are independent of one another and of what they
+  // overtake), one after the other
+  std::vector<std::vector<uint32_t>> cut;
+  schedule_list(d, list, count, &cut);
+  std::vector<trn_gemv_desc> ordered;
+  std::vector<std::pair<uint32_t, uint32_t>> ph;
+  for (const std::vector<uint32_t>& members : cut) {
+    ph.emplace_back(uint32_t(ordered.size()), uint32_t(ordered.size() + members.size()));
+    for (uint32_t mbr : members) ordered.push_back(list[mbr]);
+  }
+  const trn_gemv_desc* descs = ordered.data();
   const uint32_t phases = uint32_t(ph.size());
   std::vector<uint32_t> assign(size_t(phases) * G * 4u, 0u);   // entry, block_id, num_blocks, fmt
   std::vector<ChainEntryHost> entries(count);
@@ -551,7 +585,8 @@ hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t strea
     for (uint32_t i = 0; i < m; ++i) {
       // cost, not bytes: a Q6_K byte takes longer than a Q4_K byte (measured: the workgroups of a Q6_K entry with
       // a byte share ended 5 us after those of its Q4_K neighbours)
-      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4] * (descs[a + i].fmt == 6 ? 1.3 : 1.0);
+      const uint32_t slabs_i = std::min((descs[a + i].k / 256u + 15u) / 16u, kWaves);
+      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4] * (1.0 + 0.3 * (slabs_i - 1u));
       total += bytes[i];
     }
     // shares: at least one workgroup each, the rest in proportion to the bytes (largest remainders first)
@@ -1136,7 +1171,6 @@ trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
 }
 
 namespace {
-constexpr uint32_t kGroupMax = 8;      // entries of one grouped launch
 struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip
   ChainEntryHost e[kGroupMax];
   uint32_t first[kGroupMax + 1];
@@ -1237,42 +1271,6 @@ trn_status trn_fused_residual_rmsnorm(trn_stream s, trn_dptr residual, trn_dptr 
   return st(launch_rmsnorm(static_cast<hipStream_t>(s), residual, input, output, gamma, hidden_size, epsilon, true));
 }
 
-namespace {
-bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
-  return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
-         gemv_geometry(*dk, d.k, d.n).fits;
-}
-
-// Cuts a list into launches (mode 0).  A launch is filled with up to kGroupMax entries that are independent of one
-// another AND of every earlier entry that has not been launched yet: the first entry still waiting always goes in,
-// later ones of a window are brought forward when nothing they read or write is touched by an entry they would
-// overtake.  What an entry computes does not depend on the company it is launched in, so the results are those of
-// the list in order.
-void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches) {
-  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 16u);
-  const uint32_t group_max =
-      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupMax);
-  std::vector<uint8_t> launched(count, 0);
-  for (uint32_t pos = 0; pos < count;) {
-    if (launched[pos]) { ++pos; continue; }
-    std::vector<uint32_t> members(1, pos);
-    if (list_groupable(dk, descs[pos])) {
-      const uint32_t end = uint32_t(std::min<uint64_t>(count, uint64_t(pos) + window));
-      for (uint32_t j = pos + 1; j < end && members.size() < group_max; ++j) {
-        if (launched[j]) continue;
-        const trn_gemv_desc& c = descs[j];
-        if (!list_groupable(dk, c)) break;           // an entry that takes another path keeps its place in the order
-        bool ok = true;
-        for (uint32_t i = pos; i < j && ok; ++i)     // the members of the launch and everything it would overtake
-          if (!launched[i]) ok = !gemv_depends(c, descs[i]) && !gemv_depends(descs[i], c);
-        if (ok) members.push_back(j);
-      }
-    }
-    for (uint32_t m : members) launched[m] = 1;
-    launches->push_back(std::move(members));
-  }
-}
-}  // namespace
 
 trn_status trn_kquant_gemv_plan(const trn_gemv_desc* descs, uint32_t count, uint32_t* launch_of) {
   if (count == 0) return TRN_SUCCESS;
