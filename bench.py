@@ -299,6 +299,38 @@ def main() -> int:
             for b in bufs:
                 b.free()
 
+        # the GEMM entry points outside BASELINE's configurations: Q5_K / Q6_K (VALU engine per row of A) and the
+        # legacy 18-byte format of q4k_gemm_fused, 4096 x 4096, cold
+        n = k = 4096
+        for fmt in ("q5k", "q6k"):
+            host = kq.gen_matrix(fmt, 1239, n, k)
+            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            fn = getattr(L, f"trn_{fmt}_gemm")
+            for m in (4, 16):
+                a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
+                c = t.GpuBuffer(ctx, m * n, np.float32)
+                us = timed(lambda r: fn(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k), 2 * copies)
+                nbytes = alg_bytes(fmt, n, k) + 4 * (m - 1) * (k + n)
+                configs[f"x_{fmt}_gemm_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                                         "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+                a.free()
+                c.free()
+            for b in bufs:
+                b.free()
+        host = kq.gen_q4k_simplified(np.random.default_rng(1240), n * (k // 32))
+        bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+        for m in (1, 4):
+            a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
+            c = t.GpuBuffer(ctx, m * n, np.float32)
+            us = timed(lambda r: L.trn_q4k_gemm_fused(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k), 2 * copies)
+            nbytes = n * (k // 32) * 18 + 4 * m * (k + n)
+            configs[f"x_q4k_gemm_fused_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                                        "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            a.free()
+            c.free()
+        for b in bufs:
+            b.free()
+
     # ---- the element-wise steps between the GEMVs of a layer, one launch each (latency-bound: a few KB) ----------
     glue_us = {}
     if not args.no_configs:
