@@ -109,3 +109,48 @@ def test_entries_brought_forward_keep_the_lists_meaning(gpu, seed):
     for nm in names:
         assert np.all(np.isfinite(want[nm])), nm
         assert np.array_equal(want[nm].view(np.uint32), got[nm].view(np.uint32)), (seed, nm)
+
+
+def test_a_list_captured_into_a_hip_graph_replays_to_the_same_bits(gpu):
+    """The default way of issuing a list allocates nothing and clears nothing, so a caller may capture it into a HIP
+    graph.  Every replay, with eager launches and synchronisations in between, must give the eager result."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    ctx, stream = gpu
+    specs, x_len = CASES["layer"]
+    bufs = {"x": t.GpuBuffer.from_host(ctx, kq.gen_x(1, x_len))}
+    keep, batch = [], t.GemvBatch()
+    for i, (fmt, n, k, src, dst, flags) in enumerate(specs):
+        if dst not in bufs:
+            bufs[dst] = t.GpuBuffer.from_host(ctx, np.full(n, np.nan, np.float32))
+        w = t.GpuBuffer.from_host(ctx, kq.gen_matrix(fmt, 900 + i, n, k))
+        keep.append(w)
+        batch.add(fmt, k, n, bufs[dst], w, bufs[src], flags)
+    batch.launch(stream)                       # eager: loads the code object, gives the expected bits
+    stream.synchronize()
+    want = {nm: b.copy_to_host() for nm, b in bufs.items()}
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.raw(), 0) == 0
+    batch.launch(stream)
+    assert hip.hipStreamEndCapture(stream.raw(), C.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    try:
+        for rep in range(3):
+            for nm in bufs:
+                if nm != "x":
+                    bufs[nm].copy_from_host(np.full(len(want[nm]), np.nan, np.float32))
+            assert hip.hipGraphLaunch(gexec, stream.raw()) == 0
+            stream.synchronize()
+            for nm in bufs:
+                assert np.array_equal(bufs[nm].copy_to_host().view(np.uint32), want[nm].view(np.uint32)), (rep, nm)
+            batch.launch(stream)               # eager work between the replays
+            stream.synchronize()
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
