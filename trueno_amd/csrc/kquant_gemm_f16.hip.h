@@ -107,7 +107,7 @@ __device__ __forceinline__ void lds_write16x2(u32 addr, u32 a, u32 b) {     // t
 __device__ __forceinline__ void lds_write32(u32 addr, u32 a) { asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(a) : "memory"); }
 
 // Token operands of one super-block, written to an LDS stage of kXpStageBytes:
-//   q*1024 + (32g + 2*token + piece)*16 + 2e   f16 = piece of the scaled element 32 j + 8 (u%4) + perm[e],
+//   q*1024 + ((32g + 2*token + piece) ^ 2q)*16 + 2e   f16 = piece of the scaled element 32 j + 8 (u%4) + perm[e],
 //                                               u = q/2, h = q%2, j = 2 (2g + u/4) + h, perm = 0,2,1,3,4,6,5,7
 //   16384 + (32g + 2*token + piece)*8 + 2e     f16 = piece of 2^-5 * (sum of the scaled sub-block 4g + e)
 //   16896 + token*4                            f32 = 2^(E+14) where the run was scaled by 2^-E (NaN if the run
@@ -143,7 +143,9 @@ __device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, 
   const u32 j = c >> 2, g = j >> 2, h = j & 1u, u = 4u * ((j & 3u) >> 1) + (c & 3u), q = 2u * u + h;
   const u32x4 ph = {pack_h2(hi[0], hi[2]), pack_h2(hi[1], hi[3]), pack_h2(hi[4], hi[6]), pack_h2(hi[5], hi[7])};
   const u32x4 pl = {pack_h2(lo[0], lo[2]), pack_h2(lo[1], lo[3]), pack_h2(lo[4], lo[6]), pack_h2(lo[5], lo[7])};
-  lds_write128x2(stage + q * 1024u + (32u * g + 2u * token) * 16u, ph, pl);
+  // the 16 products' pages are 1 KB apart, i.e. on the same banks: slot s of page q lies at s ^ 2q, so that the lanes
+  // of a token, which write the same slot of different pages, do not all hit one bank (the reader applies the same)
+  lds_write128x2(stage + q * 1024u + ((32u * g + 2u * token) ^ (2u * q)) * 16u, ph, pl);
   float sj = ((xs[0] + xs[1]) + (xs[2] + xs[3])) + ((xs[4] + xs[5]) + (xs[6] + xs[7]));
   sj += dpp_f32<0xB1>(sj);
   sj += dpp_f32<0x4E>(sj);                  // the four threads of a sub-block hold its sum
@@ -236,6 +238,9 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
   f32x16 tot;
 #pragma unroll
   for (int v = 0; v < 16; ++v) tot[v] = 0.0f;
+  u32 xq[16];                                    // where this lane finds its token operands of product q (stage 0)
+#pragma unroll
+  for (u32 q = 0; q < 16; ++q) xq[q] = lds_xp + ((lane ^ (2u * q)) << 4);
 
   load_a(0);
   issue_w(0);
@@ -295,11 +300,12 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
 #pragma unroll
     for (int uu = 0; uu < 8; uu += 2) {          // two dword pairs = four products per round of operand reads
       u32x4 a0, a1, a2, a3;
+      const u32 xs = slot * kXpStageBytes;       // product q reads slot lane ^ 2q of its page (xq[q], set up once)
       switch (uu) {
-        case 0: lds_read128<0 * 1024>(a0, xl); lds_read128<1 * 1024>(a1, xl); lds_read128<2 * 1024>(a2, xl); lds_read128<3 * 1024>(a3, xl); break;
-        case 2: lds_read128<4 * 1024>(a0, xl); lds_read128<5 * 1024>(a1, xl); lds_read128<6 * 1024>(a2, xl); lds_read128<7 * 1024>(a3, xl); break;
-        case 4: lds_read128<8 * 1024>(a0, xl); lds_read128<9 * 1024>(a1, xl); lds_read128<10 * 1024>(a2, xl); lds_read128<11 * 1024>(a3, xl); break;
-        default: lds_read128<12 * 1024>(a0, xl); lds_read128<13 * 1024>(a1, xl); lds_read128<14 * 1024>(a2, xl); lds_read128<15 * 1024>(a3, xl); break;
+        case 0: lds_read128<0 * 1024>(a0, xq[0] + xs); lds_read128<1 * 1024>(a1, xq[1] + xs); lds_read128<2 * 1024>(a2, xq[2] + xs); lds_read128<3 * 1024>(a3, xq[3] + xs); break;
+        case 2: lds_read128<4 * 1024>(a0, xq[4] + xs); lds_read128<5 * 1024>(a1, xq[5] + xs); lds_read128<6 * 1024>(a2, xq[6] + xs); lds_read128<7 * 1024>(a3, xq[7] + xs); break;
+        case 4: lds_read128<8 * 1024>(a0, xq[8] + xs); lds_read128<9 * 1024>(a1, xq[9] + xs); lds_read128<10 * 1024>(a2, xq[10] + xs); lds_read128<11 * 1024>(a3, xq[11] + xs); break;
+        default: lds_read128<12 * 1024>(a0, xq[12] + xs); lds_read128<13 * 1024>(a1, xq[13] + xs); lds_read128<14 * 1024>(a2, xq[14] + xs); lds_read128<15 * 1024>(a3, xq[15] + xs); break;
       }
       const u32x4* aq[4] = {&a0, &a1, &a2, &a3};
       u32 bl[2][4], bh[2][4];
