@@ -340,13 +340,11 @@ __device__ __forceinline__ bool consume_entry(ConsumerState& st, const ChainEntr
     // stage the activation vector (coherent loads), swizzled for this format's register slices
     const u32 units = e.k >> 2;
     const u32 x_lds = st.lds_base + lay.x;
+    // the vector was written by other workgroups of this launch: 16-byte buffer loads at agent scope (sc1)
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(e.x), 0, static_cast<int>(e.k * 4u), 0x00020000);
     for (u32 u = ctid; u < units; u += cthreads) {
-      const u32* xw = reinterpret_cast<const u32*>(e.x) + 4u * u;
-      u32x4 v;
-      v.x = __hip_atomic_load(xw + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      v.y = __hip_atomic_load(xw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      v.z = __hip_atomic_load(xw + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      v.w = __hip_atomic_load(xw + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, static_cast<int>(16u * u), 0, 16);
       asm volatile("ds_write_b128 %0, %1" ::"v"(x_lds + 16u * Q::swz(u)), "v"(v) : "memory");
     }
     lds_wait();
