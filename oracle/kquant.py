@@ -20,10 +20,17 @@ How each function is pinned (the reference holds no numeric test of this path):
       independently in tests/test_oracle_pins.py (different loop structure), plus
       one-hot bit maps, closed forms, byte brute force, and the C restatement
       oracle/kquant_ref.c written separately from the same reference lines.
-  dequant_q5k, *_legacy     : only the builder calls define them.  Pinned by the
-      hand-derived scatter bit maps, closed forms and the independent C restatement;
-      no reference-held vector exists, so against the reference itself these stay
-      "parity unpinned".
+  dequant_q5k               : only the builder calls define it (no GGML equivalent).  Pinned by the
+      scatter map of all 1408 stored bits derived by hand from the cited index arithmetic, the
+      12-bit field map, closed forms, exactness (fp64-then-round == f32) and the C restatement.
+  dequant_q4k/q5k/q6k_legacy: only the builder calls define them.  Pinned by hand-derived scatter
+      maps of every quant bit (sequential nibbles qs[i//2]; B' fifth bit i%8 of qh[i//8]; C'
+      ql[i//2], qh[i//4] with weight 4, unsigned scale i//16), one-field-at-a-time scale/min
+      selection, closed forms (zero quants, all-ones quants), the visible difference between the
+      uncontracted sequence (the definition here) and a fused multiply-subtract, and the C
+      restatement.  Each of these fails under a swapped nibble, a wrong weight, a wrong scale
+      packing or a signed/unsigned slip.  No reference-held vector exists for any decode, so
+      nothing here is checked against a running reference.
   gemv_fp64 / gemm_fp64     : closed form (an fp64 dot product), brute force on tiny shapes.
   gemv_ref_order_fp32       : emulation of the reference's lane/summation order; used only
       to compare error magnitudes, never for bit parity.

@@ -232,6 +232,144 @@ def test_q6k_scale_map_and_sign():
         assert np.array_equal(wl, expect_l), sidx
 
 
+# ---- GEMM-family ("legacy", as written) decodes A', B', C' ---------------------------------------
+# quantize.rs:445-514 (A'), :727-807 (B'), :1009-1064 (C').  What the cited index arithmetic fixes, derived by hand:
+#   A'/B': sub-block j = i // 32 reads its (scale, min) from the 12-bit field j; value i = 32 j + lane reads
+#          qs[16 j + lane // 2] = qs[i // 2], low nibble for even i (:488-507); B' adds bit i % 8 of qh[i // 8]
+#          at byte 144, weight 16 (:781-795); scale and min are multiplied by rn(1/63) first (:477-482).
+#   C'   : 16 sub-blocks of 16; value i reads ql[i // 2] (nibble i & 1), bits 2 (i % 4) of qh[i // 4] at byte 128
+#          with weight FOUR (q = ql + 4 qh - 32, :1051-1057), scale = unsigned byte 192 + i // 16.
+def _unit_block_legacy(fmt):
+    """d = 1 (dmin = 1), every scale field at the value that normalises to exactly 1: w = q - 1 (A', B'), q - 32 (C')"""
+    blk = np.zeros(kq.SB_BYTES[fmt], np.uint8)
+    if fmt == "q6k":
+        blk[192:208] = 1
+        blk[208:210] = f16(1.0)
+        return blk
+    blk[0:2] = f16(1.0)
+    blk[2:4] = f16(1.0)
+    blk[4:16] = 0xFF          # s_j = m_j = 63, and rn(63 * rn(1/63)) == 1 (asserted below)
+    return blk
+
+
+def _quant_bit_map_legacy(fmt):
+    m = {}
+    if fmt in ("q4k", "q5k"):
+        for B in range(128):           # qs byte B holds values 2B (low nibble) and 2B + 1 (high nibble)
+            for b in range(8):
+                m[(16 + B, b)] = (2 * B + b // 4, 1 << (b % 4))
+        if fmt == "q5k":
+            for B in range(32):
+                for b in range(8):
+                    m[(144 + B, b)] = (8 * B + b, 16)
+    else:
+        for B in range(128):           # ql byte B: values 2B, 2B + 1
+            for b in range(8):
+                m[(B, b)] = (2 * B + b // 4, 1 << (b % 4))
+        for B in range(64):            # qh byte B: values 4B .. 4B + 3, two bits each, weight 4 (not 16)
+            for b in range(8):
+                m[(128 + B, b)] = (4 * B + b // 2, 4 << (b % 2))
+    return m
+
+
+def test_inv63_normalises_63_to_one():
+    inv63 = np.float32(1.0) / np.float32(63.0)
+    assert np.float32(63.0) * inv63 == np.float32(1.0)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_scatter_bit_map_legacy(fmt, co):
+    base_blk = _unit_block_legacy(fmt)
+    base = kq.DEQUANT[(fmt, 1)](base_blk)[0]
+    offset = -32.0 if fmt == "q6k" else -1.0
+    assert np.all(base == offset)
+    bitmap = _quant_bit_map_legacy(fmt)
+    n_quant_bits = {"q4k": 128 * 8, "q5k": 160 * 8, "q6k": 192 * 8}[fmt]
+    assert len(bitmap) == n_quant_bits
+    keys = sorted(bitmap)
+    blocks = np.tile(base_blk, (n_quant_bits, 1))
+    for row, (byte, bit) in enumerate(keys):
+        blocks[row, byte] |= 1 << bit
+    w = kq.DEQUANT[(fmt, 1)](blocks.reshape(-1))
+    assert np.array_equal(bits(w), bits(co.dequant(fmt, blocks.reshape(-1), 1)))
+    for row, key in enumerate(keys):
+        idx, inc = bitmap[key]
+        expect = np.full(256, offset, np.float32)
+        expect[idx] += inc
+        assert np.array_equal(w[row], expect), (fmt, key)
+    # the legacy map is NOT the GEMV-family one: the same one-hot blocks decode differently under policy 0
+    w0 = kq.DEQUANT[(fmt, 0)](blocks.reshape(-1))
+    assert not np.array_equal(np.argmax(w0 != w0[:, :1], axis=1), np.argmax(w != w[:, :1], axis=1))
+
+
+@pytest.mark.parametrize("fmt", ("q4k", "q5k"))
+def test_legacy_scale_and_min_select_subblock(fmt):
+    """A'/B': field j governs values 32 j .. 32 j + 31.  One field at a time: with q = 1 everywhere and dmin = 0,
+    w = rn(d * rn(s * rn(1/63))); with q = 0, w = -rn(dmin * rn(m * rn(1/63)))."""
+    F = np.float32
+    inv63 = F(1.0) / F(63.0)
+    d, dmin = F(np.float16(0.0173)), F(np.float16(0.0081))
+    for j in range(8):
+        for kind in ("s", "m"):
+            val = 37 + j
+            field = val << (12 * j + (0 if kind == "s" else 6))
+            blk = np.zeros(kq.SB_BYTES[fmt], np.uint8)
+            blk[0:2] = f16(d)
+            blk[2:4] = f16(dmin)
+            blk[4:16] = np.frombuffer(field.to_bytes(12, "little"), np.uint8)
+            blk[16:144] = 0x11
+            w = kq.DEQUANT[(fmt, 1)](blk)[0]
+            expect = np.zeros(256, np.float32)
+            if kind == "s":
+                expect[32 * j:32 * j + 32] = F(F(d * F(F(val) * inv63)) * F(1.0))
+            else:
+                expect[32 * j:32 * j + 32] = F(F(0.0) - F(dmin * F(F(val) * inv63)))
+            assert np.array_equal(bits(w), bits(expect)), (fmt, j, kind)
+
+
+def test_legacy_q6k_closed_forms():
+    """C': all-zero quants -> rn(d * sc) * (-32) with the UNSIGNED scale of sub-block i // 16; qh weighs 4:
+    ql = 15 and q2 = 3 give q = 15 + 12 - 32 = -5 (the GEMV-family decode would give 63 - 32 = 31)."""
+    F = np.float32
+    blk = kq.gen_q6k(np.random.default_rng(77), 8).reshape(8, 210).copy()
+    blk[:, :192] = 0
+    w = kq.dequant_q6k_legacy(blk.reshape(-1))
+    d = np.array([f32_of_f16(b[208:210]) for b in blk], np.float32)
+    sc = blk[:, 192:208].astype(np.float32)                     # unsigned
+    expect = np.repeat((d[:, None] * sc).astype(F), 16, axis=1) * F(-32.0)
+    assert np.array_equal(bits(w), bits(expect))
+    blk[:, :192] = 0xFF
+    w = kq.dequant_q6k_legacy(blk.reshape(-1))
+    assert np.array_equal(bits(w), bits(np.repeat((d[:, None] * sc).astype(F), 16, axis=1) * F(-5.0)))
+    assert np.array_equal(bits(kq.dequant_q6k(blk.reshape(-1))[:, :1]),
+                          bits((d * blk[:, 192].view(np.int8).astype(F))[:, None] * F(31.0)))
+
+
+@pytest.mark.parametrize("fmt", ("q4k", "q5k"))
+def test_legacy_contraction_ambiguity_is_visible(fmt):
+    """A'/B' are inexact: the sequence mul, mul, sub (the definition used here) and the sequence in which the last
+    mul and the sub are one fused multiply-add differ on some values, and never by more than one rounding."""
+    F = np.float32
+    inv63 = F(1.0) / F(63.0)
+    blk = kq.GEN[fmt](np.random.default_rng(91), 64).reshape(64, -1)
+    w = kq.DEQUANT[(fmt, 1)](blk.reshape(-1))
+    d = np.array([f32_of_f16(b[0:2]) for b in blk], F)
+    dmin = np.array([f32_of_f16(b[2:4]) for b in blk], F)
+    s, m = kq.scales_mins_12bit(blk[:, 4:16])
+    ds = np.repeat((d[:, None] * (s.astype(F) * inv63)).astype(F), 32, axis=1)
+    dm = np.repeat((dmin[:, None] * (m.astype(F) * inv63)).astype(F), 32, axis=1)
+    q = np.empty((64, 256), np.float64)
+    q[:, 0::2] = blk[:, 16:144] & 15
+    q[:, 1::2] = blk[:, 16:144] >> 4
+    if fmt == "q5k":
+        q += 16.0 * np.unpackbits(blk[:, 144:176], axis=1, bitorder="little")
+    fused = (ds.astype(np.float64) * q - dm.astype(np.float64)).astype(F)     # exact product, one rounding
+    differ = bits(fused) != bits(w)
+    assert differ.any() and not differ.all()
+    ulp = np.spacing(np.maximum(np.abs(w), np.abs(fused)).astype(F))
+    assert np.all(np.abs(w.astype(np.float64) - fused.astype(np.float64)) <= 2.0 * ulp.astype(np.float64) + 2.0 * np.spacing(np.abs(ds * q.astype(F)).astype(F)))
+
+
 # ---- closed forms -----------------------------------------------------------------------------
 @pytest.mark.parametrize("fmt", ("q4k", "q5k"))
 def test_closed_form_zero_quants(fmt):
