@@ -230,7 +230,7 @@ def main() -> int:
 
     # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
     other_modes = {}
-    for mode, label in (() if args.no_executors else ((1, "resident_phases"), (2, "streaming_producer"))):
+    for mode, label in (() if args.no_executors else ((1, "resident_phases"),)):
         L.trn_set_tuning(b"batch_mode", mode)
         ms, _ = run_passes(max(3, args.steps // 2), 1)
         other_modes[label] = round(ms * 1e3, 1)

@@ -44,6 +44,11 @@ typedef struct trn_event_s* trn_event;
 #define TRN_ERROR_NO_DEVICE 100         /* hipErrorNoDevice */
 #define TRN_ERROR_INVALID_DEVICE 101    /* hipErrorInvalidDevice */
 #define TRN_ERROR_NOT_FOUND 500         /* hipErrorNotFound */
+/* Not a hipError_t: a device-side wait of the resident list executor (batch_mode 1) ran out of its spin budget and
+ * the kernel gave up.  Reported once, by the next trn_stream_synchronize / trn_event_synchronize /
+ * trn_ctx_synchronize / trn_stream_destroy / trn_kquant_gemv_batch on that stream; the outputs of that list are
+ * not valid.  The context stays usable. */
+#define TRN_ERROR_WAIT_ABANDONED 9001
 #define TRN_STREAM_NON_BLOCKING 1u      /* CU_STREAM_NON_BLOCKING, driver/stream.rs:60 */
 
 /* ---- 1. initialisation (sys.rs:101-102) ------------------------------------------------ */
@@ -67,6 +72,16 @@ TRN_API trn_status trn_module_load_data(trn_module* module, const void* image); 
 TRN_API trn_status trn_module_unload(trn_module module);                        /* cuModuleUnload */
 TRN_API trn_status trn_module_get_function(trn_function* func, trn_module module,
                                            const char* name);                   /* cuModuleGetFunction */
+/* The reference compiles some kernel parameters into the PTX of one kernel instance: RmsNormKernel::new(hidden_size)
+ * .with_epsilon(e) (layernorm.rs:388-431), FusedResidualRmsNormKernel (elementwise.rs:109-149) and
+ * IncrementalAttentionKernel::new / ::with_gqa (attention.rs:808-901).  A pre-built code object cannot, so they are
+ * set on the function handle (one module per kernel instance, as in the reference) before it is launched by name with
+ * the reference's own parameter list: "rmsnorm" (input, output, gamma), "fused_residual_rmsnorm" (residual, input,
+ * output, gamma), "incremental_attention" (q, k, v, out, seq_len).  Launching one of these by name without its
+ * constants returns TRN_ERROR_INVALID_VALUE; nothing beyond the reference's parameters is ever read. */
+TRN_API trn_status trn_function_set_rmsnorm(trn_function func, uint32_t hidden_size, float epsilon);
+TRN_API trn_status trn_function_set_attention(trn_function func, uint32_t head_dim, uint32_t num_heads,
+                                              uint32_t num_kv_heads, uint32_t max_seq_len, float scale);
 
 /* ---- 5. memory (sys.rs:142-176) ------------------------------------------------------------ */
 TRN_API trn_status trn_mem_alloc(trn_dptr* ptr, size_t size);                   /* cuMemAlloc_v2 */
@@ -87,7 +102,10 @@ TRN_API trn_status trn_stream_synchronize(trn_stream stream);                   
  * (driver/stream.rs:110-154).  For the k-quant kernels of the built-in module the grid, block and
  * shared-memory arguments are ignored and replaced by the kernel's own geometry (the reference's
  * documented grid = N blocks of 32 threads, quantize.rs:1151-1155, is a warp32 shape); the result
- * never depends on the geometry the caller passed.  Other functions launch exactly as given. */
+ * never depends on the geometry the caller passed.  The same holds for a module made by trn_module_load_data from
+ * the image trn_builtin_image returns.  Kernels of the built-in code object that are not reference names are
+ * internal: launching one by name returns TRN_ERROR_INVALID_VALUE.  Functions of any other module launch exactly
+ * as given. */
 TRN_API trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y, unsigned grid_z,
                                      unsigned block_x, unsigned block_y, unsigned block_z,
                                      unsigned shared_mem_bytes, trn_stream stream,
@@ -101,7 +119,8 @@ TRN_API trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigne
  *   q4k_gemm_ggml         q5k_gemm_ggml         q6k_gemm_ggml          (a, b_quant, c, m, n, k)
  *   q4k_gemm_fused                                                      (a, b_quant, c, m, n, k) */
 TRN_API trn_status trn_module_load_builtin(trn_module* module);
-/* Pointer to and size of that embedded code object (for callers that want trn_module_load_data). */
+/* Pointer to and size of that embedded code object (for callers that want trn_module_load_data; the module is
+ * recognised and treated like trn_module_load_builtin's). */
 TRN_API trn_status trn_builtin_image(const void** image, size_t* size);
 
 /* ---- 8. typed launchers ------------------------------------------------------------------------
@@ -134,14 +153,13 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * entry still waiting, plus later ones of a window of the list (q, k, v of a decoder layer; gate and up; ...)
  * that depend neither on it nor on anything they would overtake.  What an entry computes does not depend on the
  * company it is launched in: the results are, bit for bit, those of one launch per entry in list order.
- * With trn_set_tuning("batch_mode", 1 or 2), and when every entry meets the fast kernels' alignment (x 16 B,
+ * With trn_set_tuning("batch_mode", 1), and when every entry meets the fast kernels' alignment (x 16 B,
  * W 16 B / 2 B for Q6_K), the list runs as ONE cooperative launch of resident workgroups: the list is cut in
- * phases of mutually independent entries with a device-side barrier between phases (mode 1), or a producer wave
- * per CU streams the weights through an LDS ring (mode 2).  These forms keep, per (device, stream), small device
- * buffers with the list, the work assignment and the barrier counters (allocated on first use, kept until the
- * stream is destroyed); a list identical to the previous one on that stream is not uploaded again.  If a device-side
- * wait ever runs out of its (seconds-long) spin budget the kernel exits and the next call on that stream returns
- * hipErrorLaunchFailure (719).  All three forms give bit-identical results. */
+ * phases of mutually independent entries with a device-side barrier between phases.  This form keeps, per
+ * (device, stream), small device buffers with the list, the work assignment and the barrier counters (allocated on
+ * first use, kept until the stream is destroyed); a list identical to the previous one on that stream is not uploaded
+ * again.  If a device-side wait ever runs out of its (seconds-long) spin budget the kernel exits and the next
+ * synchronising call on that stream returns TRN_ERROR_WAIT_ABANDONED.  Both forms give bit-identical results. */
 /* An entry may fold the element-wise steps of a decoder layer in (zero pointers: absent):
  *   x'  = x                          or silu(x) * x2            (TRN_GEMV_SWIGLU_INPUT; x = gate, x2 = up: fused_swiglu)
  *   x'' = x' * gamma                 (gamma: k f32, the weights of rmsnorm)
@@ -192,7 +210,8 @@ TRN_API trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event st
  *   q, out: [num_heads][head_dim] f32;  k, v: [num_kv_heads][max_seq_len][head_dim] f32.
  * trueno-gpu/src/kernels/attention.rs:808-1095 (IncrementalAttentionKernel, "incremental_attention", parameters
  * (q_ptr, k_ptr, v_ptr, out_ptr, seq_len); head_dim, the head counts, max_seq_len and scale are compiled into its
- * PTX and follow as parameters here, also in a by-name launch).  The reference's kernel covers head_dim <= 64;
+ * PTX: here they are arguments of the typed launcher, and constants of the function handle for a by-name launch,
+ * trn_function_set_attention).  The reference's kernel covers head_dim <= 64;
  * this one head_dim % 4 == 0 up to 256.  1 <= seq_len <= max_seq_len; pointers 16-byte aligned.  Keeps a small
  * per-stream workspace (allocated on first use). */
 TRN_API trn_status trn_incremental_attention(trn_stream stream, trn_dptr q, trn_dptr k, trn_dptr v, trn_dptr out,
@@ -213,9 +232,9 @@ TRN_API trn_status trn_gemv_f32(trn_stream stream, trn_dptr y, trn_dptr a, trn_d
 
 /* ---- element-wise steps between the GEMVs of a decoder layer (f32 vectors) ---------------------------------
  * The same kernels are in the built-in module under the reference's names "residual_add", "fused_swiglu",
- * "rmsnorm", "fused_residual_rmsnorm".  The first two keep the reference's parameter lists; the reference
- * compiles hidden_size and epsilon of the two norms into its PTX, here they follow the pointers as two more
- * parameters (u32 hidden_size, f32 epsilon).  Whatever grid and block a by-name launch passes is replaced. */
+ * "rmsnorm", "fused_residual_rmsnorm", all with the reference's parameter lists.  The reference compiles hidden_size
+ * and epsilon of the two norms into its PTX; for a by-name launch they are constants of the function handle
+ * (trn_function_set_rmsnorm).  Whatever grid and block a by-name launch passes is replaced. */
 /* output[i] = input1[i] + input2[i]; output may alias an input.  trueno-gpu/src/kernels/elementwise.rs:33-101 */
 TRN_API trn_status trn_residual_add(trn_stream stream, trn_dptr input1, trn_dptr input2, trn_dptr output, uint32_t n);
 /* output[i] = silu(gate[i]) * up[i], silu(g) = g / (1 + 2^(-g * 1.442695f)).  elementwise.rs:521-592 */
@@ -235,11 +254,9 @@ TRN_API const char* trn_error_name(trn_status status);
 TRN_API const char* trn_error_string(trn_status status);
 /* Number of compute units of the current device (sizes the launches). */
 TRN_API trn_status trn_device_cu_count(int* count);
-/* Launch tuning knobs, process-wide; 0 restores the default.  "gemv_blocks_per_cu", "gemv_row_groups":
- * geometry of the single-GEMV kernels.  "batch_mode": how trn_kquant_gemv_batch runs a list - 0 one
- * launch per entry (default), 1 one cooperative launch of resident workgroups with device-side
- * barriers, 2 as 1 with a producer wave per CU streaming the weights through an LDS ring.
- * "stream_consumers": consumer waves of mode 2.
+/* Launch tuning knobs, process-wide (for tests and measurements; atomics, no other synchronisation); 0 restores the default.  "gemv_blocks_per_cu", "gemv_row_groups":
+ * geometry of the single-GEMV kernels.  "batch_mode": how trn_kquant_gemv_batch runs a list - 0 grouped
+ * launches (default), 1 one cooperative launch of resident workgroups with device-side barriers.
  * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
  * "group_off": 1 = in mode 0 one launch per entry; "group_max": most entries in a launch (0 = 8); "group_window":
  * how far down the list a launch looks for entries (0 = 16); "group_slab_weight": percent added to an entry's

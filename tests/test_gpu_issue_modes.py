@@ -1,6 +1,5 @@
-"""GPU parity, streaming form of the list executor (producer wave + LDS ring): must give the same bits
-as the one-launch-per-entry path for every format, ragged row counts, shares larger than the ring and
-K > 4096 (several waves per row)."""
+"""GPU parity of the three ways a list is issued (grouped launches, one launch per entry, resident phases): the
+same bits for every format, ragged row counts and K > 4096 (several waves per row)."""
 import numpy as np
 import pytest
 
@@ -51,7 +50,7 @@ CASES = {
 
 
 @pytest.mark.parametrize("case", sorted(CASES))
-def test_stream_equals_per_entry_launches(gpu, case):
+def test_issue_modes_give_the_same_bits(gpu, case):
     specs, x_len = CASES[case]
     ctx, _ = gpu
     # inputs named g0/d0 are extra seeded vectors
@@ -61,9 +60,9 @@ def test_stream_equals_per_entry_launches(gpu, case):
     if case == "q5k_mixed":
         specs2[-1] = ("q5k", 4096, 1024, "x", "e", 0)
     ref = _run(gpu, specs2, x_len, {"batch_mode": 0})
-    got = _run(gpu, specs2, x_len, {"batch_mode": 2})
+    got = _run(gpu, specs2, x_len, {"group_off": 1})
     for name in ref:
-        assert np.array_equal(ref[name].view(np.uint32), got[name].view(np.uint32)), (case, name)
+        assert np.array_equal(ref[name].view(np.uint32), got[name].view(np.uint32)), (case, name, "one launch per entry")
     old = _run(gpu, specs2, x_len, {"batch_mode": 1})
     for name in ref:
         assert np.array_equal(ref[name].view(np.uint32), old[name].view(np.uint32)), (case, name, "resident phases")

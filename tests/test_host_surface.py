@@ -136,3 +136,18 @@ def test_no_device_error_convention():
     assert L.trn_q4k_gemv(None, 16, 16, 16, 256, 4) == 100       # would launch: no device
     assert L.trn_mem_free(0) == 0
     assert L.trn_set_tuning(b"no_such_key", 1) == 1
+
+
+def test_argument_checks_that_need_no_device():
+    L = _ffi.lib()
+    assert L.trn_function_set_rmsnorm(None, 4096, 1e-5) == 1           # no function handle
+    assert L.trn_function_set_attention(None, 128, 32, 32, 2048, 0.1) == 1
+    assert L.trn_set_tuning(b"batch_mode", 2) == 1                      # 0 = grouped launches, 1 = resident phases, nothing else
+    assert L.trn_set_tuning(b"batch_mode", 0) == 0
+    assert L.trn_error_name(9001) == b"TRN_ERROR_WAIT_ABANDONED"
+    # a list is validated as a whole before the device is touched: the bad entry is the LAST one
+    good = _ffi.GemvDesc(4, 256, 0, 0, 16, 16, 16, 0, 0, 0, 0.0, 0)     # n = 0: a no-op entry
+    bad = _ffi.GemvDesc(4, 100, 4, 0, 16, 16, 16, 0, 0, 0, 0.0, 0)      # k % 256 != 0
+    assert L.trn_kquant_gemv_batch(None, (_ffi.GemvDesc * 2)(good, bad), 2) == 1
+    null_y = _ffi.GemvDesc(4, 256, 4, 0, 0, 16, 16, 0, 0, 0, 0.0, 0)
+    assert L.trn_kquant_gemv_batch(None, (_ffi.GemvDesc * 2)(good, null_y), 2) == 1

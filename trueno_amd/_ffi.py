@@ -27,6 +27,8 @@ SIGNATURES = {
     "trn_module_load_data": [C.POINTER(vp), vp],
     "trn_module_unload": [vp],
     "trn_module_get_function": [C.POINTER(vp), vp, C.c_char_p],
+    "trn_function_set_rmsnorm": [vp, C.c_uint32, C.c_float],
+    "trn_function_set_attention": [vp, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_float],
     "trn_mem_alloc": [C.POINTER(dptr), C.c_size_t],
     "trn_mem_free": [dptr],
     "trn_memcpy_htod": [dptr, vp, C.c_size_t],

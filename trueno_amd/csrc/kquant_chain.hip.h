@@ -28,12 +28,6 @@
 #pragma once
 #include "kquant_quarter.hip.h"
 
-// CHAIN_STAMP(slot): a hook for timing probes (0 start, 1 after the barrier wait, 2 activations staged, 4 after the
-// sum of squares, 5 after the row loop, 3 end); a probe defines it before including this file.
-#ifndef CHAIN_STAMP
-#define CHAIN_STAMP(slot) do { } while (0)
-#endif
-
 // One GEMV of a list with the element-wise steps of a decoder layer folded in:
 //   x'  = x                         or  silu(x) * x2                         (CHAIN_SWIGLU_INPUT; fused_swiglu)
 //   x'' = x' * gamma                (gamma != null)
@@ -125,6 +119,9 @@ template <int FMT, int U, bool COHERENT = false>
 __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
                                            f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks) {
   using Q = Quarter<FMT>;
+  // The engine is built for whole waves: a block that is not a positive multiple of 64 threads (the reference's own
+  // geometry is 32) would divide by zero below and never leave the staging loop.  Uniform exit before any barrier.
+  if (blockDim.x < 64u || (blockDim.x & 63u) != 0u) return true;
   const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;
@@ -139,8 +136,6 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   const bool wave_active = grp < groups && grp < batches;
   const u32 sbl = lane >> 2, c = lane & 3u;
   const size_t row_bytes = static_cast<size_t>(nsb) * Q::SB;
-
-  CHAIN_STAMP(0);
   typename Q::Regs regs[U];
   auto issue = [&](u32 slab, u32 b) {
     const u32 sb = slab * 16u + sbl;
@@ -202,7 +197,6 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
 
   if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
   if (polls) issue(sw, wave_active ? grp : 0u);
-  CHAIN_STAMP(1);
   if (!has_rows) return true;
 
   float* part = reinterpret_cast<float*>(lds4 + units);
@@ -236,14 +230,12 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   __shared__ u32 s_next[16];
   if (tid < 16u) s_next[tid] = groups;
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  CHAIN_STAMP(2);
   float scale = 1.0f;
   if (norm) {
     float total = group_ss[0];
     for (u32 g = 1; g < xgroups; ++g) total += group_ss[g];
     scale = 1.0f / sqrtf(total / static_cast<float>(k_dim) + (e.eps != 0.0f ? e.eps : kChainNormEps));
   }
-  CHAIN_STAMP(4);
 
   if (wave_active) {
     for (u32 slab = sw; slab < slabs; slab += sw_count) {
@@ -283,7 +275,6 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
       }
     }
   }
-  CHAIN_STAMP(5);
   __syncthreads();
   for (u32 t = tid; t < rows_per_block; t += blockDim.x) {
     const u32 row = row0 + t;
@@ -302,7 +293,6 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
       }
     }
   }
-  CHAIN_STAMP(3);
   return true;
 }
 

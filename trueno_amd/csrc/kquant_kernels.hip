@@ -12,7 +12,6 @@
 #define KQ_U 2      // rows a wave of the fast GEMV engine has in flight (the host's kGemvRowsPerBatch)
 #endif
 #include "kquant_chain.hip.h"
-#include "kquant_stream.hip.h"
 #include "kquant_gemm_f16.hip.h"
 #include "decode_glue.hip.h"
 #include "gemv_f32.hip.h"
@@ -112,13 +111,6 @@ extern "C" __global__ void __launch_bounds__(768) kq_gemv_group(const GemvGroup 
 extern "C" __global__ void __launch_bounds__(768)
 kq_gemv_phases(const ChainEntry* entries, const PhaseAssign* assign, u32 phases, u32* counters, u32* status, u32 spin_limit) {
   phases_body<KQ_U>(entries, assign, phases, counters, status, spin_limit);
-}
-
-// The list with decoupled weight streaming (kquant_stream.hip.h): one workgroup per CU.
-extern "C" __global__ void __launch_bounds__(512)
-kq_gemv_stream(const ChainEntry* entries, u32 count, u32* counters, u32* status, u32 spin_limit, u32 x_bytes_max,
-               u32 rows_max, u32 slabs_max) {
-  stream::stream_body(entries, count, counters, status, spin_limit, x_bytes_max, rows_max, slabs_max);
 }
 
 // ------------------------------------------------------------------------------------------

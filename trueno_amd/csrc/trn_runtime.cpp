@@ -11,6 +11,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstdio>
 #include <cstring>
@@ -43,8 +44,11 @@ const char* const kFmtName[NFMT] = {"q4k", "q5k", "q6k"};
 const uint32_t kSbBytes[NFMT] = {144, 176, 210};
 
 // kinds of functions the launch-by-name path recognises
+// KIND_OTHER: a function of a caller's own code object, launched exactly as given.  KIND_INTERNAL: a kernel of the
+// built-in code object that is not one of the reference's names; its geometry and extra arguments belong to the
+// typed entry points, so a by-name launch of it is refused.
 enum Kind { KIND_OTHER = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GEMM_SIMPLIFIED = 3, KIND_RESIDUAL_ADD = 4, KIND_SWIGLU = 5,
-            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8, KIND_ATTENTION = 9 };
+            KIND_RMSNORM = 6, KIND_RESIDUAL_RMSNORM = 7, KIND_GEMV_F32 = 8, KIND_ATTENTION = 9, KIND_INTERNAL = 10 };
 
 constexpr int kMaxDevices = 64;
 #ifndef KQ_U
@@ -54,16 +58,13 @@ constexpr uint32_t kGemvRowsPerBatch = KQ_U;  // U of the fast GEMV kernel (the 
 constexpr uint32_t kGemvMaxWaves = 12;        // __launch_bounds__(768) of the fast GEMV kernels
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
-constexpr uint32_t kFlagNormInput = 1u, kFlagBarrierBefore = 2u, kFlagSameX = 4u;   // CHAIN_* of kquant_chain.hip.h
-// kquant_stream.hip.h: control block, ring (+16 mirror bytes), activations, partial sums, counters
-constexpr uint32_t kStreamCtlBytes = 256, kStreamRingBytes = 96 * 1024, kStreamLdsLimit = 160 * 1024 - 1024;
 
 struct DeviceKernels {
   bool loaded = false;
   hipModule_t module = nullptr;
   int cu_count = 0;
   hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
-  hipFunction_t stream = nullptr, fill_u32 = nullptr, gemv_group = nullptr, phases = nullptr;
+  hipFunction_t fill_u32 = nullptr, gemv_group = nullptr, phases = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
@@ -76,21 +77,22 @@ struct DeviceKernels {
 };
 
 std::mutex g_mutex;
+// The tuning knobs are process-wide and meant for tests and measurements: atomics, so that a thread that flips one
+// while another launches is a race on the setting, never on memory.
 DeviceKernels g_dev[kMaxDevices];
-int g_tune_blocks_per_cu = 0;
-int g_tune_row_groups = 0;
-int g_tune_batch_mode = 0;   // 0: launches (default); 1: resident phases + barriers; 2: resident, streaming producer wave
-int g_tune_chain_spin_limit = 0;
-int g_tune_stream_consumers = 0;
-int g_tune_group_off = 0;
-int g_tune_gemm_mfma_off = 0;   // 1: the Q4_K GEMM never takes the matrix-core form
-int g_tune_gemm_ksplit = 0;     // parts of K in the matrix-core GEMM (0: chosen from the shape)
-int g_tune_attention_min_steps = 0;
-int g_tune_group_window = 0;       // entries of a list a grouped launch may look ahead over (0: 16)
-int g_tune_group_max = 0;          // most entries in one grouped launch (0: 8)
-int g_tune_slab_weight = 0;        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
-int g_tune_attention_per_cu = 0;   // workgroups per CU the single-query attention aims at (0: default)
-int g_tune_gemm_waves = 0;      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
+std::atomic<int> g_tune_blocks_per_cu{0};
+std::atomic<int> g_tune_row_groups{0};
+std::atomic<int> g_tune_batch_mode{0};   // 0: launches (default); 1: resident phases + barriers
+std::atomic<int> g_tune_chain_spin_limit{0};
+std::atomic<int> g_tune_group_off{0};
+std::atomic<int> g_tune_gemm_mfma_off{0};   // 1: the Q4_K GEMM never takes the matrix-core form
+std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
+std::atomic<int> g_tune_attention_min_steps{0};
+std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped launch may look ahead over (0: 16)
+std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8)
+std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
+std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
+std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -139,7 +141,6 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.swiglu, "fused_swiglu")) != hipSuccess ||
         (e = get_fn(m, &t.rmsnorm, "rmsnorm")) != hipSuccess ||
         (e = get_fn(m, &t.residual_rmsnorm, "fused_residual_rmsnorm")) != hipSuccess ||
-        (e = get_fn(m, &t.stream, "kq_gemv_stream")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
         (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
@@ -242,13 +243,45 @@ hipError_t launch_rmsnorm(hipStream_t stream, uint64_t residual, uint64_t in, ui
   return hipModuleLaunchKernel(d->rmsnorm, 1, 1, 1, block, 1, 1, 0, stream, args, nullptr);
 }
 
-// f32 GEMV y = A^T-style product with A K x N row-major (gemv_f32.hip.h).  Partial results of the parts of K and
-// the arrival counters live in a per-(device, stream) buffer like the GEMM's.
-struct GemvF32Workspace {
+// Per-(device, stream) scratch buffers of the kernels that cut their work in parts (partial results + arrival
+// counters at the front).  g_ws_mutex is held across lookup, growth and the launch that zeroes new counters, so two
+// threads on two streams never see a half-grown buffer; a buffer only ever belongs to one stream, and work on one
+// stream is ordered, so the kernels themselves need no lock.  New counters are zeroed by a small fill kernel, not by
+// hipMemsetAsync: the call may be recorded into a HIP graph by a capturing caller.
+struct ScratchWorkspace {
   void* buf = nullptr;
   size_t cap = 0;
 };
-std::map<std::pair<int, hipStream_t>, GemvF32Workspace> g_gemv_f32_ws;
+using ScratchMap = std::map<std::pair<int, hipStream_t>, ScratchWorkspace>;
+std::mutex g_ws_mutex;
+
+hipError_t acquire_scratch(ScratchMap& map, DeviceKernels* d, hipStream_t stream, size_t need, size_t zero_bytes, uint64_t* base) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  ScratchWorkspace& ws = map[std::make_pair(dev, stream)];
+  if (ws.cap < need) {
+    if (ws.buf) {
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;   // work in flight may still use the old buffer
+      (void)hipFree(ws.buf);
+      ws.buf = nullptr;
+      ws.cap = 0;
+    }
+    if ((e = hipMalloc(&ws.buf, need)) != hipSuccess) return e;
+    ws.cap = need;
+    uint32_t words = uint32_t(zero_bytes / 4u), zero = 0u;
+    void* fill_args[] = {&ws.buf, &words, &zero};
+    const uint32_t grid = std::max(1u, std::min(64u, (words + 255u) / 256u));
+    if ((e = hipModuleLaunchKernel(d->fill_u32, grid, 1, 1, 256, 1, 1, 0, stream, fill_args, nullptr)) != hipSuccess) return e;
+  }
+  *base = reinterpret_cast<uint64_t>(ws.buf);
+  return hipSuccess;
+}
+
+// f32 GEMV y = A^T-style product with A K x N row-major (gemv_f32.hip.h).  Partial results of the parts of K and
+// the arrival counters live in a per-(device, stream) buffer like the GEMM's.
+ScratchMap g_gemv_f32_ws;
 
 hipError_t launch_gemv_f32(hipStream_t stream, uint64_t y, uint64_t a, uint64_t x, uint32_t k, uint32_t n) {
   if (n == 0) return hipSuccess;
@@ -269,32 +302,16 @@ hipError_t launch_gemv_f32(hipStream_t stream, uint64_t y, uint64_t a, uint64_t 
   parts = (k + rows_per_part - 1u) / rows_per_part;
   const size_t cnt_cap = 64u * 1024u, need = cnt_cap + (parts > 1u ? size_t(parts) * n * 4u : 0u);
   if (size_t(tiles) * 4u > cnt_cap) return hipErrorInvalidValue;
-  int dev = 0;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-  GemvF32Workspace* ws;
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    ws = &g_gemv_f32_ws[std::make_pair(dev, stream)];
-  }
-  if (ws->cap < need) {
-    if (ws->buf) {
-      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;
-      (void)hipFree(ws->buf);
-      ws->buf = nullptr;
-      ws->cap = 0;
-    }
-    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
-    ws->cap = need;
-    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;   // the kernel leaves the counters at zero
-  }
-  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  uint64_t cnt = 0;
+  if ((e = acquire_scratch(g_gemv_f32_ws, d, stream, need, cnt_cap, &cnt)) != hipSuccess) return e;   // the kernel leaves the counters at zero
+  uint64_t part = cnt + cnt_cap;
   void* args[] = {&y, &a, &x, &part, &cnt, &k, &n, &rows_per_part, &parts};
   return hipModuleLaunchKernel(d->gemv_f32_fast, tiles * parts, 1, 1, 512, 1, 1, 0, stream, args, nullptr);
 }
 
 // Single-query attention over the KV cache (decode_attention.hip.h).  Per (device, stream): arrival counters per
 // head and the chunks' partial softmax states.
-std::map<std::pair<int, hipStream_t>, GemvF32Workspace> g_attention_ws;
+ScratchMap g_attention_ws;
 
 hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t v, uint64_t out, uint32_t seq_len,
                             uint32_t head_dim, uint32_t num_heads, uint32_t num_kv_heads, uint32_t max_seq_len, float scale) {
@@ -319,25 +336,9 @@ hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t
   chunk = (chunk + step - 1u) / step * step;
   chunks = (seq_len + chunk - 1u) / chunk;
   const size_t cnt_cap = 64u * 1024u, need = cnt_cap + (chunks > 1u ? size_t(num_heads) * chunks * lpp * 32u : 0u);
-  int dev = 0;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-  GemvF32Workspace* ws;
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    ws = &g_attention_ws[std::make_pair(dev, stream)];
-  }
-  if (ws->cap < need) {
-    if (ws->buf) {
-      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;
-      (void)hipFree(ws->buf);
-      ws->buf = nullptr;
-      ws->cap = 0;
-    }
-    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
-    ws->cap = need;
-    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;   // the kernel leaves the counters at zero
-  }
-  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  uint64_t cnt = 0;
+  if ((e = acquire_scratch(g_attention_ws, d, stream, need, cnt_cap, &cnt)) != hipSuccess) return e;   // the kernel leaves the counters at zero
+  uint64_t part = cnt + cnt_cap;
   void* args[] = {&q, &k, &v, &out, &seq_len, &head_dim, &num_heads, &num_kv_heads, &max_seq_len, &scale, &lpp_log2, &chunk, &chunks,
                   &part, &cnt};
   return hipModuleLaunchKernel(d->attention, num_heads * chunks, 1, 1, 256, 1, 1, 0, stream, args, nullptr);
@@ -345,16 +346,15 @@ hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t
 
 // Partial results and arrival counters of the matrix-core GEMM: one buffer per (device, stream), grown on
 // demand and kept.  The counters are zero between products: the kernel puts them back.
-struct GemmWorkspace {
-  void* buf = nullptr;
-  size_t cap = 0;
-};
-std::map<std::pair<int, hipStream_t>, GemmWorkspace> g_gemm_ws;
+ScratchMap g_gemm_ws;
 
 constexpr uint32_t kGemmXpStageBytes = 16 * 1024 + 512 + 64, kGemmWTileBytes = 32 * 144;
+constexpr size_t kGemmCounterBytes = size_t(1) << 16;   // arrival counters at the front of the GEMM's scratch buffer
 
+// ext_base != 0: the caller brings the scratch buffer (ext_cap bytes, counters at its front already zero); nothing is
+// allocated and a product that needs more is refused.
 hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
-                               uint32_t n, uint32_t k) {
+                               uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
   // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
   const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
@@ -370,33 +370,28 @@ hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a,
   const size_t cnt_bytes = up(size_t(groups) * tiles * 4u);
   // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
   const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * groups * waves * 2048u) : 0u;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  GemmWorkspace* ws;
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    ws = &g_gemm_ws[std::make_pair(dev, stream)];
-  }
-  // the counters sit at the end of a region that only grows, so a larger product finds zeros there too
-  const size_t cnt_cap = up(size_t(1) << 16), need = cnt_cap + part_bytes;
+  // the counters sit at the front of a region that only grows, so a larger product finds zeros there too (the
+  // kernel puts every counter it used back to zero)
+  const size_t cnt_cap = kGemmCounterBytes, need = cnt_cap + part_bytes;
   if (cnt_bytes > cnt_cap) return hipErrorInvalidValue;
-  if (ws->cap < need) {
-    if (ws->buf) {
-      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return e;   // a GEMM in flight may still use it
-      (void)hipFree(ws->buf);
-      ws->buf = nullptr;
-      ws->cap = 0;
-    }
-    if ((e = hipMalloc(&ws->buf, need)) != hipSuccess) return e;
-    ws->cap = need;
-    if ((e = hipMemsetAsync(ws->buf, 0, cnt_cap, stream)) != hipSuccess) return e;
+  uint64_t cnt = ext_base;
+  if (ext_base != 0) {
+    if (need > ext_cap) return hipErrorInvalidValue;
+  } else {
+    hipError_t e = acquire_scratch(g_gemm_ws, d, stream, need, cnt_cap, &cnt);
+    if (e != hipSuccess) return e;
   }
-  uint64_t cnt = reinterpret_cast<uint64_t>(ws->buf), part = cnt + cnt_cap;
+  uint64_t part = cnt + cnt_cap;
   const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
   uint32_t nsb_arg = nsb, ksb_arg = ksb, kparts_arg = kparts, groups_arg = groups, tiles_arg = tiles;
   void* margs[] = {&a, &w, &c, &part, &cnt, &m, &n, &nsb_arg, &ksb_arg, &kparts_arg, &groups_arg, &tiles_arg};
   return hipModuleLaunchKernel(d->gemm_f16[waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
+}
+
+// does the matrix-core form take this product?
+bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  return m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
+         uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u;   // its arrival counters
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
@@ -407,9 +402,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
-  if (!is_gemv && f == Q4K && m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
-      uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u)   // its arrival counters
-    return launch_q4k_gemm_f16(d, stream, a, w, c, m, n, k);
+  if (!is_gemv && f == Q4K && q4k_gemm_f16_ok(a, w, c, m, n, k)) return launch_q4k_gemm_f16(d, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
@@ -689,31 +682,10 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
     if (g.n == 0 || g.k == 0 || !g.x || !g.w || !g.y) return hipSuccess;
     if (!gemv_fast_ok(Fmt(g.fmt - 4), g.y, g.w, g.x)) return hipSuccess;
   }
-  // entries: barrier where an entry touches what an entry of the current group wrote (or overwrites
-  // what one of them reads)
-  std::vector<ChainEntryHost> entries(count);
-  uint32_t barriers = 0;
-  size_t group_begin = 0;
-  for (uint32_t i = 0; i < count; ++i) {
-    const trn_gemv_desc& g = descs[i];
-    bool dep = false;
-    for (size_t j = group_begin; j < i && !dep; ++j) {
-      const trn_gemv_desc& p = descs[j];
-      dep = desc_conflict(g, p);
-    }
-    if (dep) {
-      ++barriers;
-      group_begin = i;
-    }
-    entries[i] = entry_of(g, dep ? kFlagBarrierBefore : 0u);
-  }
   int dev = 0;
-  (void)hipGetDevice(&dev);
-  ChainWorkspace* ws;
-  {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    ws = &g_chain_ws[std::make_pair(dev, stream)];
-  }
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);   // across the workspace's growth, the uploads and the launch
+  ChainWorkspace* ws = &g_chain_ws[std::make_pair(dev, stream)];
   if (!ws->h_status) {
     if ((e = hipHostMalloc(reinterpret_cast<void**>(&ws->h_status), 64, hipHostMallocMapped)) != hipSuccess) return e;
     ws->h_status[0] = 0;
@@ -721,83 +693,7 @@ hipError_t launch_chain(hipStream_t stream, const trn_gemv_desc* descs, uint32_t
   }
   if (ws->h_status[0] != 0) {  // an earlier list on this stream gave up at a wait: report it once
     ws->h_status[0] = 0;
-    return hipErrorLaunchFailure;
-  }
-
-  if (g_tune_batch_mode != 2) return launch_phases(d, ws, stream, descs, count, handled);
-
-  // ---- streaming form: one workgroup per CU, a producer wave feeding an LDS ring -------------------
-  bool use_stream = g_tune_batch_mode == 2;
-  for (uint32_t i = 0; i < count; ++i) use_stream = use_stream && !desc_extended(descs[i]);   // the streaming kernel has no folded steps
-  uint32_t consumers = g_tune_stream_consumers > 0 ? uint32_t(g_tune_stream_consumers) : 7u;
-  consumers = std::max(1u, std::min(consumers, 7u));
-  const uint32_t sgrid = uint32_t(d->cu_count);
-  uint32_t x_bytes_max = 0, rows_max = 1, slabs_max = 1;
-  for (uint32_t i = 0; i < count && use_stream; ++i) {
-    const trn_gemv_desc& g = descs[i];
-    const uint32_t nsb = g.k / 256u, slabs = (nsb + 15u) / 16u;
-    const uint64_t row_bytes = uint64_t(nsb) * kSbBytes[g.fmt - 4];
-    const uint64_t rows = (uint64_t(g.n) + sgrid - 1) / sgrid;
-    if (slabs > consumers || (uint64_t(g.n) * row_bytes) % 16u != 0 || rows * row_bytes >= (1ull << 31)) use_stream = false;
-    x_bytes_max = std::max<uint32_t>(x_bytes_max, g.k * 4u);
-    slabs_max = std::max(slabs_max, slabs);
-    if (slabs > 1) rows_max = std::max<uint32_t>(rows_max, uint32_t(rows));
-  }
-  uint32_t slds = kStreamCtlBytes + kStreamRingBytes + 16u + x_bytes_max + rows_max * slabs_max * 4u + rows_max * 4u;
-  if (slds > kStreamLdsLimit) use_stream = false;
-  if (use_stream) {
-    // entries that read the same vector (same length, same register layout) as their predecessor,
-    // with no barrier in between, keep the activations where they are
-    for (uint32_t i = 1; i < count; ++i) {
-      const bool q6a = descs[i].fmt == 6, q6b = descs[i - 1].fmt == 6;
-      if (!(entries[i].flags & kFlagBarrierBefore) && descs[i].x == descs[i - 1].x && descs[i].k == descs[i - 1].k && q6a == q6b)
-        entries[i].flags |= kFlagSameX;
-    }
-  }
-  auto upload = [&](uint32_t grid_for_counters) -> hipError_t {
-    const bool same = ws->last.size() == entries.size() &&
-                      std::memcmp(ws->last.data(), entries.data(), entries.size() * sizeof(ChainEntryHost)) == 0;
-    if (!same) {
-      hipError_t err = hipStreamSynchronize(stream);  // the device copy may still be read by a list in flight
-      if (err != hipSuccess) return err;
-      if (ws->cap_entries < entries.size()) {
-        if (ws->d_entries) (void)hipFree(ws->d_entries);
-        ws->d_entries = nullptr;
-        ws->cap_entries = 0;
-        if ((err = hipMalloc(&ws->d_entries, entries.size() * sizeof(ChainEntryHost))) != hipSuccess) return err;
-        ws->cap_entries = entries.size();
-      }
-      if ((err = hipMemcpy(ws->d_entries, entries.data(), entries.size() * sizeof(ChainEntryHost), hipMemcpyHostToDevice)) != hipSuccess)
-        return err;
-      ws->last = entries;
-    }
-    const size_t n_words = size_t(barriers + 1u) * chain_barrier_stride_host(grid_for_counters);
-    if (ws->cap_counters < n_words) {
-      hipError_t err = hipStreamSynchronize(stream);
-      if (err != hipSuccess) return err;
-      if (ws->d_counters) (void)hipFree(ws->d_counters);
-      ws->d_counters = nullptr;
-      ws->cap_counters = 0;
-      if ((err = hipMalloc(reinterpret_cast<void**>(&ws->d_counters), n_words * sizeof(uint32_t))) != hipSuccess) return err;
-      ws->cap_counters = n_words;
-    }
-    uint32_t n_counters = uint32_t(n_words), zero = 0u;
-    void* fill_args[] = {&ws->d_counters, &n_counters, &zero};
-    const uint32_t fill_grid = std::max(1u, std::min(64u, (n_counters + 255u) / 256u));
-    return hipModuleLaunchKernel(d->fill_u32, fill_grid, 1, 1, 256, 1, 1, 0, stream, fill_args, nullptr);
-  };
-  uint32_t spin_limit = g_tune_chain_spin_limit > 0 ? uint32_t(g_tune_chain_spin_limit) : 4000000u;
-  uint32_t cnt = count;
-  if (use_stream) {
-    if ((e = upload(sgrid)) != hipSuccess) return e;
-    void* args[] = {&ws->d_entries, &cnt, &ws->d_counters, &ws->d_status, &spin_limit, &x_bytes_max, &rows_max, &slabs_max};
-    e = hipModuleLaunchCooperativeKernel(d->stream, sgrid, 1, 1, 64u * (1u + consumers), 1, 1, slds, stream, args);
-    if (e == hipSuccess) {
-      ws->grid = sgrid; ws->block = 64u * (1u + consumers); ws->lds = slds; ws->barriers = barriers;
-      *handled = true;
-      return hipSuccess;
-    }
-    (void)hipGetLastError();   // not launchable in this form here: try the plain resident form below
+    return static_cast<hipError_t>(TRN_ERROR_WAIT_ABANDONED);
   }
 
   return launch_phases(d, ws, stream, descs, count, handled);
@@ -812,6 +708,12 @@ struct trn_function_s {
   hipFunction_t fn;
   int kind;
   int fmt;
+  // what the reference compiles into the PTX of one kernel instance (trn_function_set_rmsnorm / _set_attention)
+  bool has_constants;
+  uint32_t hidden_size;
+  float epsilon;
+  uint32_t head_dim, num_heads, num_kv_heads, max_seq_len;
+  float scale;
 };
 struct trn_module_s {
   hipModule_t module;
@@ -821,6 +723,7 @@ struct trn_module_s {
 };
 struct trn_event_s {
   hipEvent_t ev;
+  hipStream_t stream;   // where it was recorded last
 };
 
 namespace {
@@ -891,16 +794,46 @@ trn_status trn_ctx_set_current(trn_ctx ctx) {
   return st(hipSetDevice(ctx->device));
 }
 
-trn_status trn_ctx_synchronize(void) { return st(hipDeviceSynchronize()); }
+trn_status trn_ctx_synchronize(void) {
+  TRN_TRY(hipDeviceSynchronize());
+  int dev = 0;
+  TRN_TRY(hipGetDevice(&dev));
+  trn_status waited = TRN_SUCCESS;      // every stream of the device is idle now: report (once) any abandoned wait
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  for (auto& kv : g_chain_ws)
+    if (kv.first.first == dev && kv.second.h_status && kv.second.h_status[0] != 0) {
+      kv.second.h_status[0] = 0;
+      waited = TRN_ERROR_WAIT_ABANDONED;
+    }
+  return waited;
+}
 
 // ---- 4. modules --------------------------------------------------------------------------
+// Is `image` (an ELF code object in host memory) a copy of the built-in one?  The length comes from the image's own
+// ELF header (section header table at the end), so nothing is read beyond what the loader itself would read.
+static bool image_is_builtin(const void* image) {
+  if (image == static_cast<const void*>(trn_builtin_hsaco_begin)) return true;
+  const unsigned char* p = static_cast<const unsigned char*>(image);
+  const size_t builtin_size = size_t(trn_builtin_hsaco_end - trn_builtin_hsaco_begin);
+  if (builtin_size < 64 || std::memcmp(p, trn_builtin_hsaco_begin, 64) != 0) return false;   // Elf64_Ehdr, e_shoff included
+  uint64_t shoff;
+  uint16_t shentsize, shnum;
+  std::memcpy(&shoff, p + 40, 8);
+  std::memcpy(&shentsize, p + 58, 2);
+  std::memcpy(&shnum, p + 60, 2);
+  const uint64_t elf_size = shoff + uint64_t(shentsize) * shnum;
+  return elf_size <= builtin_size && elf_size >= 64 && std::memcmp(p, trn_builtin_hsaco_begin, size_t(elf_size)) == 0;
+}
+
 trn_status trn_module_load_data(trn_module* module, const void* image) {
   if (!module || !image) return TRN_ERROR_INVALID_VALUE;
   hipModule_t m = nullptr;
   TRN_TRY(hipModuleLoadData(&m, image));
   trn_module_s* h = new trn_module_s();
   h->module = m;
-  h->builtin = false;
+  // the built-in image handed back through trn_builtin_image gets the same treatment as trn_module_load_builtin:
+  // its kernels keep their own geometry however the caller launches them
+  h->builtin = image_is_builtin(image);
   *module = h;
   return TRN_SUCCESS;
 }
@@ -941,8 +874,9 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
   }
   hipFunction_t f = nullptr;
   TRN_TRY(hipModuleGetFunction(&f, module->module, name));
-  trn_function_s* h = new trn_function_s{f, KIND_OTHER, 0};
+  trn_function_s* h = new trn_function_s{f, KIND_OTHER, 0, false, 0u, 0.0f, 0u, 0u, 0u, 0u, 0.0f};
   if (module->builtin) {
+    h->kind = KIND_INTERNAL;
     const std::string n = name;
     for (int i = 0; i < NFMT; ++i) {
       if (n == std::string(kFmtName[i]) + "_gemv_warp_reduce") { h->kind = KIND_GEMV; h->fmt = i; }
@@ -958,6 +892,26 @@ trn_status trn_module_get_function(trn_function* func, trn_module module, const 
   }
   module->functions[name] = h;
   *func = h;
+  return TRN_SUCCESS;
+}
+
+trn_status trn_function_set_rmsnorm(trn_function func, uint32_t hidden_size, float epsilon) {
+  if (!func || (func->kind != KIND_RMSNORM && func->kind != KIND_RESIDUAL_RMSNORM) || !(epsilon >= 0.0f)) return TRN_ERROR_INVALID_VALUE;
+  func->hidden_size = hidden_size;
+  func->epsilon = epsilon;
+  func->has_constants = true;
+  return TRN_SUCCESS;
+}
+
+trn_status trn_function_set_attention(trn_function func, uint32_t head_dim, uint32_t num_heads, uint32_t num_kv_heads,
+                                      uint32_t max_seq_len, float scale) {
+  if (!func || func->kind != KIND_ATTENTION) return TRN_ERROR_INVALID_VALUE;
+  func->head_dim = head_dim;
+  func->num_heads = num_heads;
+  func->num_kv_heads = num_kv_heads;
+  func->max_seq_len = max_seq_len;
+  func->scale = scale;
+  func->has_constants = true;
   return TRN_SUCCESS;
 }
 
@@ -1031,7 +985,7 @@ trn_status trn_stream_create(trn_stream* stream, unsigned flags) {
 // The per-(device, stream) scratch buffers of a stream that is going away (partial sums, arrival counters, the
 // resident executor's tables).  The stream must be idle.
 static void release_stream_workspaces(hipStream_t stream) {
-  std::lock_guard<std::mutex> lock(g_mutex);
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto drop_simple = [&](auto& map) {
     for (auto it = map.begin(); it != map.end();) {
       if (it->first.second == stream) {
@@ -1059,17 +1013,35 @@ static void release_stream_workspaces(hipStream_t stream) {
   }
 }
 
+// A resident executor whose device-side wait ran out of its spin budget leaves a mark in the stream's status word and
+// exits; the work behind it on the stream still runs, on stale data.  Every call that tells the caller "the stream's
+// work is done" looks at the word, clears it and reports TRN_ERROR_WAIT_ABANDONED once.
+static trn_status take_wait_status(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return TRN_SUCCESS;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_chain_ws.find(std::make_pair(dev, stream));
+  if (it == g_chain_ws.end() || !it->second.h_status || it->second.h_status[0] == 0) return TRN_SUCCESS;
+  it->second.h_status[0] = 0;
+  return TRN_ERROR_WAIT_ABANDONED;
+}
+
 trn_status trn_stream_destroy(trn_stream stream) {
   if (!stream) return TRN_ERROR_INVALID_VALUE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // work that still uses the stream's scratch buffers must have finished before they are freed
   const hipError_t e = hipStreamSynchronize(s);
+  const trn_status waited = take_wait_status(s);
   release_stream_workspaces(s);
   const hipError_t d = hipStreamDestroy(s);
-  return st(e != hipSuccess ? e : d);
+  if (e != hipSuccess) return st(e);
+  return d != hipSuccess ? st(d) : waited;
 }
 
-trn_status trn_stream_synchronize(trn_stream stream) { return st(hipStreamSynchronize(static_cast<hipStream_t>(stream))); }
+trn_status trn_stream_synchronize(trn_stream stream) {
+  TRN_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return take_wait_status(static_cast<hipStream_t>(stream));
+}
 
 trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned block_x,
                              unsigned block_y, unsigned block_z, unsigned shared_mem_bytes, trn_stream stream,
@@ -1097,17 +1069,17 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     if (func->kind == KIND_GEMM_SIMPLIFIED) return st(launch_gemm_simplified(s, p0, p1, p2, m, n, k));
     return st(launch_gemm_like(Fmt(func->fmt), s, p0, p1, p2, m, n, k, false));
   }
-  if (func->kind == KIND_ATTENTION) {      // (q, k, v, out, seq_len), then head_dim, num_heads, num_kv_heads, max_seq_len, scale
-    if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
-    for (int i = 0; i < 10; ++i)
+  if (func->kind == KIND_INTERNAL) return TRN_ERROR_INVALID_VALUE;   // only the typed entry points launch these
+  if (func->kind == KIND_ATTENTION) {      // (q_ptr, k_ptr, v_ptr, out_ptr, seq_len): attention.rs:897-901, nothing beyond
+    if (!kernel_params || !func->has_constants) return TRN_ERROR_INVALID_VALUE;
+    for (int i = 0; i < 5; ++i)
       if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
     uint64_t p[4];
-    uint32_t u[5];
-    float scale;
+    uint32_t seq_len;
     for (int i = 0; i < 4; ++i) std::memcpy(&p[i], kernel_params[i], 8);
-    for (int i = 0; i < 5; ++i) std::memcpy(&u[i], kernel_params[4 + i], 4);
-    std::memcpy(&scale, kernel_params[9], 4);
-    return st(launch_attention(s, p[0], p[1], p[2], p[3], u[0], u[1], u[2], u[3], u[4], scale));
+    std::memcpy(&seq_len, kernel_params[4], 4);
+    return st(launch_attention(s, p[0], p[1], p[2], p[3], seq_len, func->head_dim, func->num_heads, func->num_kv_heads,
+                               func->max_seq_len, func->scale));
   }
   if (func->kind == KIND_GEMV_F32) {                                           // (y, a, x, k_dim, n_dim)
     if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
@@ -1132,19 +1104,17 @@ trn_status trn_launch_kernel(trn_function func, unsigned grid_x, unsigned grid_y
     std::memcpy(&n, kernel_params[3], 4);
     return st(launch_elementwise(Kind(func->kind), s, p0, p1, p2, n));
   }
-  if (func->kind == KIND_RMSNORM || func->kind == KIND_RESIDUAL_RMSNORM) {     // pointers, then hidden_size, epsilon
+  if (func->kind == KIND_RMSNORM || func->kind == KIND_RESIDUAL_RMSNORM) {
+    // (input, output, gamma) layernorm.rs:426-428 / (residual, input, output, gamma) elementwise.rs:146-149; the row
+    // length and epsilon are constants of the kernel instance (trn_function_set_rmsnorm), never read from the array
     const int np = func->kind == KIND_RMSNORM ? 3 : 4;
-    if (!kernel_params) return TRN_ERROR_INVALID_VALUE;
-    for (int i = 0; i < np + 2; ++i)
+    if (!kernel_params || !func->has_constants) return TRN_ERROR_INVALID_VALUE;
+    for (int i = 0; i < np; ++i)
       if (!kernel_params[i]) return TRN_ERROR_INVALID_VALUE;
     uint64_t p[4] = {0, 0, 0, 0};
     for (int i = 0; i < np; ++i) std::memcpy(&p[i], kernel_params[i], 8);
-    uint32_t hidden;
-    float eps;
-    std::memcpy(&hidden, kernel_params[np], 4);
-    std::memcpy(&eps, kernel_params[np + 1], 4);
-    if (np == 3) return st(launch_rmsnorm(s, 0, p[0], p[1], p[2], hidden, eps, false));
-    return st(launch_rmsnorm(s, p[0], p[1], p[2], p[3], hidden, eps, true));
+    if (np == 3) return st(launch_rmsnorm(s, 0, p[0], p[1], p[2], func->hidden_size, func->epsilon, false));
+    return st(launch_rmsnorm(s, p[0], p[1], p[2], p[3], func->hidden_size, func->epsilon, true));
   }
   return st(hipModuleLaunchKernel(func->fn, grid_x, grid_y, grid_z, block_x, block_y, block_z, shared_mem_bytes, s,
                                   kernel_params, extra));
@@ -1198,7 +1168,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   // further slab of 4096 columns; "group_slab_weight" overrides the percentage).
   auto cost_of = [&](const trn_gemv_desc& e) {
     const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
-    const double per_slab = (g_tune_slab_weight > 0 ? g_tune_slab_weight : 30) / 100.0;
+    const double per_slab = (g_tune_slab_weight > 0 ? int(g_tune_slab_weight) : 30) / 100.0;
     return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
   };
   for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
@@ -1288,17 +1258,24 @@ trn_status trn_kquant_gemv_plan(const trn_gemv_desc* descs, uint32_t count, uint
 trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint32_t count) {
   if (count == 0) return TRN_SUCCESS;
   if (!descs) return TRN_ERROR_INVALID_VALUE;
-  for (uint32_t i = 0; i < count; ++i)  // validate the whole list before anything is launched
-    if (descs[i].fmt < 4 || descs[i].fmt > 6 || (descs[i].flags & ~(TRN_GEMV_NORM_INPUT | TRN_GEMV_SWIGLU_INPUT)) != 0 ||
-        descs[i].k % 256u != 0 || ((descs[i].flags & TRN_GEMV_SWIGLU_INPUT) != 0) != (descs[i].x2 != 0) ||
-        !aligned(descs[i].gamma, 16) || !aligned(descs[i].x2, 16) || !aligned(descs[i].residual, 4) || !(descs[i].norm_eps >= 0.0f))
+  for (uint32_t i = 0; i < count; ++i) {  // the whole list is validated before anything is launched
+    const trn_gemv_desc& g = descs[i];
+    if (g.fmt < 4 || g.fmt > 6 || (g.flags & ~(TRN_GEMV_NORM_INPUT | TRN_GEMV_SWIGLU_INPUT)) != 0 || g.k % 256u != 0 ||
+        ((g.flags & TRN_GEMV_SWIGLU_INPUT) != 0) != (g.x2 != 0) || !aligned(g.gamma, 16) || !aligned(g.x2, 16) ||
+        !aligned(g.residual, 4) || !(g.norm_eps >= 0.0f))
       return TRN_ERROR_INVALID_VALUE;
+    if (g.n != 0 && ((g.k != 0 && (!g.x || !g.w)) || !g.y)) return TRN_ERROR_INVALID_VALUE;
+  }
+  DeviceKernels* dk = nullptr;
+  hipError_t e = device_kernels(&dk);
+  if (e != hipSuccess) return st(e);
+  for (uint32_t i = 0; i < count; ++i)
+    // folded element-wise steps need the fast engine (x, x2, gamma 16-byte aligned; the vector and a row block in LDS)
+    if (desc_extended(descs[i]) && !list_groupable(dk, descs[i])) return TRN_ERROR_INVALID_VALUE;
   hipStream_t stream = static_cast<hipStream_t>(s);
   bool handled = false;
-  hipError_t e = launch_chain(stream, descs, count, &handled);
+  e = launch_chain(stream, descs, count, &handled);
   if (handled || e != hipSuccess) return st(e);
-  DeviceKernels* dk = nullptr;
-  if ((e = device_kernels(&dk)) != hipSuccess) return st(e);
   std::vector<std::vector<uint32_t>> launches;
   schedule_list(dk, descs, count, &launches);
   std::vector<trn_gemv_desc> group;
@@ -1308,9 +1285,6 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
       group.clear();
       for (uint32_t m : members) group.push_back(descs[m]);
       e = launch_gemv_group(dk, stream, group.data(), uint32_t(group.size()));
-    } else if (desc_extended(head)) {
-      // folded element-wise steps need the fast engine (x, x2, gamma 16-byte aligned; the vector and a row block in LDS)
-      return TRN_ERROR_INVALID_VALUE;
     } else {
       e = launch_gemm_like(Fmt(head.fmt - 4), stream, head.x, head.w, head.y, 1, head.n, head.k, true, head.flags);
     }
@@ -1335,7 +1309,7 @@ trn_status trn_event_create(trn_event* event) {
   if (!event) return TRN_ERROR_INVALID_VALUE;
   hipEvent_t e = nullptr;
   TRN_TRY(hipEventCreate(&e));
-  *event = new trn_event_s{e};
+  *event = new trn_event_s{e, nullptr};
   return TRN_SUCCESS;
 }
 
@@ -1348,12 +1322,14 @@ trn_status trn_event_destroy(trn_event event) {
 
 trn_status trn_event_record(trn_event event, trn_stream stream) {
   if (!event) return TRN_ERROR_INVALID_VALUE;
+  event->stream = static_cast<hipStream_t>(stream);
   return st(hipEventRecord(event->ev, static_cast<hipStream_t>(stream)));
 }
 
 trn_status trn_event_synchronize(trn_event event) {
   if (!event) return TRN_ERROR_INVALID_VALUE;
-  return st(hipEventSynchronize(event->ev));
+  TRN_TRY(hipEventSynchronize(event->ev));
+  return take_wait_status(event->stream);
 }
 
 trn_status trn_event_elapsed_ms(float* ms, trn_event start, trn_event stop) {
@@ -1373,8 +1349,14 @@ trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t
   return st(hipModuleLaunchKernel(d->copy_u128, grid, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(stream), args, nullptr));
 }
 
-const char* trn_error_name(trn_status status) { return hipGetErrorName(static_cast<hipError_t>(status)); }
-const char* trn_error_string(trn_status status) { return hipGetErrorString(static_cast<hipError_t>(status)); }
+const char* trn_error_name(trn_status status) {
+  if (status == TRN_ERROR_WAIT_ABANDONED) return "TRN_ERROR_WAIT_ABANDONED";
+  return hipGetErrorName(static_cast<hipError_t>(status));
+}
+const char* trn_error_string(trn_status status) {
+  if (status == TRN_ERROR_WAIT_ABANDONED) return "TRN_ERROR_WAIT_ABANDONED: a device-side wait of the resident list executor gave up";
+  return hipGetErrorString(static_cast<hipError_t>(status));
+}
 
 trn_status trn_device_cu_count(int* count) {
   if (!count) return TRN_ERROR_INVALID_VALUE;
@@ -1388,9 +1370,12 @@ trn_status trn_set_tuning(const char* key, int value) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!std::strcmp(key, "gemv_blocks_per_cu")) { g_tune_blocks_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_row_groups")) { g_tune_row_groups = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "batch_mode")) { g_tune_batch_mode = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "batch_mode")) {
+    if (value > 1) return TRN_ERROR_INVALID_VALUE;
+    g_tune_batch_mode = value;
+    return TRN_SUCCESS;
+  }
   if (!std::strcmp(key, "chain_spin_limit")) { g_tune_chain_spin_limit = value; return TRN_SUCCESS; }
-  if (!std::strcmp(key, "stream_consumers")) { g_tune_stream_consumers = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }

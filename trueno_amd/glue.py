@@ -2,9 +2,10 @@
 ResidualAddKernel, FusedSwigluKernel, RmsNormKernel, FusedResidualRmsNormKernel - and of its f32 GEMV kernels
 (kernels/gemv.rs): GemvKernel, CoalescedGemvKernel.
 
-Constructors, fields, `name()` strings and pointer parameter order are the reference's.  The reference compiles
-`hidden_size` and `epsilon` of the two norms into the PTX it emits; the pre-built kernels here take them as two
-more parameters after the pointers, which `kernel_args()` appends.
+Constructors, fields, `name()` strings and parameter lists are the reference's.  The reference compiles
+`hidden_size` and `epsilon` of the two norms (and the shape of the attention kernel) into the PTX of one kernel
+instance; with a pre-built code object they are constants of the function handle, which `launch_by_name()` sets
+(trn_function_set_rmsnorm / trn_function_set_attention) before it launches with the reference's own arguments.
 """
 from __future__ import annotations
 
@@ -80,14 +81,16 @@ class RmsNormKernel(Kernel):
         return LaunchConfig((1, 1, 1), (32, 1, 1), 0)
 
     def kernel_args(self, input, output, gamma):
-        return [C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma)), C.c_uint32(self.hidden_size),
-                C.c_float(self.epsilon)]
+        """(input_ptr, output_ptr, gamma_ptr) - layernorm.rs:426-428."""
+        return [C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma))]
 
     def launch(self, stream: CudaStream, input, output, gamma) -> None:
         _check(_lib().trn_rmsnorm(stream.raw() if stream is not None else None, _ptr(input), _ptr(output), _ptr(gamma),
                                   self.hidden_size, self.epsilon), "KernelLaunch", self.name())
 
     def launch_by_name(self, stream: CudaStream, module: CudaModule, input, output, gamma) -> None:
+        _check(_lib().trn_function_set_rmsnorm(module.get_function(self.name()), self.hidden_size, self.epsilon),
+               "KernelLaunch", self.name())
         stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(input, output, gamma))
 
 
@@ -109,8 +112,8 @@ class FusedResidualRmsNormKernel(Kernel):
         return LaunchConfig((1, 1, 1), (32, 1, 1), 0)
 
     def kernel_args(self, residual, input, output, gamma):
-        return [C.c_uint64(_ptr(residual)), C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma)),
-                C.c_uint32(self.hidden_size), C.c_float(self.epsilon)]
+        """(residual_ptr, input_ptr, output_ptr, gamma_ptr) - elementwise.rs:146-149."""
+        return [C.c_uint64(_ptr(residual)), C.c_uint64(_ptr(input)), C.c_uint64(_ptr(output)), C.c_uint64(_ptr(gamma))]
 
     def launch(self, stream: CudaStream, residual, input, output, gamma) -> None:
         _check(_lib().trn_fused_residual_rmsnorm(stream.raw() if stream is not None else None, _ptr(residual), _ptr(input),
@@ -118,6 +121,8 @@ class FusedResidualRmsNormKernel(Kernel):
                "KernelLaunch", self.name())
 
     def launch_by_name(self, stream: CudaStream, module: CudaModule, residual, input, output, gamma) -> None:
+        _check(_lib().trn_function_set_rmsnorm(module.get_function(self.name()), self.hidden_size, self.epsilon),
+               "KernelLaunch", self.name())
         stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(residual, input, output, gamma))
 
 
@@ -186,10 +191,8 @@ class IncrementalAttentionKernel(Kernel):
         return LaunchConfig((self.num_heads, 1, 1), (32, 1, 1), 0)
 
     def kernel_args(self, q, k, v, out, seq_len: int):
-        """(q_ptr, k_ptr, v_ptr, out_ptr, seq_len) - attention.rs:897-901 - then what the reference compiles in."""
-        return [C.c_uint64(_ptr(q)), C.c_uint64(_ptr(k)), C.c_uint64(_ptr(v)), C.c_uint64(_ptr(out)), C.c_uint32(seq_len),
-                C.c_uint32(self.head_dim), C.c_uint32(self.num_heads), C.c_uint32(self.num_kv_heads),
-                C.c_uint32(self.max_seq_len), C.c_float(self.scale)]
+        """(q_ptr, k_ptr, v_ptr, out_ptr, seq_len) - attention.rs:897-901."""
+        return [C.c_uint64(_ptr(q)), C.c_uint64(_ptr(k)), C.c_uint64(_ptr(v)), C.c_uint64(_ptr(out)), C.c_uint32(seq_len)]
 
     def launch(self, stream: CudaStream, q, k, v, out, seq_len: int) -> None:
         _check(_lib().trn_incremental_attention(stream.raw() if stream is not None else None, _ptr(q), _ptr(k), _ptr(v), _ptr(out),
@@ -197,4 +200,6 @@ class IncrementalAttentionKernel(Kernel):
                                                 self.scale), "KernelLaunch", self.name())
 
     def launch_by_name(self, stream: CudaStream, module: CudaModule, q, k, v, out, seq_len: int) -> None:
+        _check(_lib().trn_function_set_attention(module.get_function(self.name()), self.head_dim, self.num_heads,
+                                                 self.num_kv_heads, self.max_seq_len, self.scale), "KernelLaunch", self.name())
         stream.launch_kernel(module, self.name(), self.launch_config(), self.kernel_args(q, k, v, out, seq_len))
