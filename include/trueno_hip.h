@@ -49,6 +49,9 @@ typedef struct trn_event_s* trn_event;
  * trn_ctx_synchronize / trn_stream_destroy / trn_kquant_gemv_batch on that stream; the outputs of that list are
  * not valid.  The context stays usable. */
 #define TRN_ERROR_WAIT_ABANDONED 9001
+/* Not a hipError_t: trn_q4k_gemm_noalloc was asked for a product whose partial results do not fit the library's
+ * static scratch buffer.  Nothing was launched. */
+#define TRN_ERROR_SCRATCH_TOO_SMALL 9002
 #define TRN_STREAM_NON_BLOCKING 1u      /* CU_STREAM_NON_BLOCKING, driver/stream.rs:60 */
 
 /* ---- 1. initialisation (sys.rs:101-102) ------------------------------------------------ */
@@ -138,6 +141,19 @@ TRN_API trn_status trn_q6k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_d
 TRN_API trn_status trn_q4k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q5k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+
+/* trn_q4k_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results; but where trn_q4k_gemm keeps a per-stream scratch buffer that it allocates and grows on demand (partial
+ * results of the parts of K and their arrival counters), this entry point uses a buffer that is part of the library
+ * image: a static device array of 8 MiB + 64 KiB, of which every GPU the library runs on holds one copy until the
+ * process ends.  After the library's first use on the device (any launcher, or trn_ctx_set_current, loads the kernels
+ * and looks the buffer's address up once) it calls nothing that allocates or frees.  A product that needs more
+ * scratch than that returns TRN_ERROR_SCRATCH_TOO_SMALL and launches nothing (every shape up to 1.5 x the CU count
+ * of 16-token x 256-row tiles fits; m = 1 and unaligned operands take kernels that need no scratch).  All calls on
+ * one GPU share that GPU's buffer: calls that overlap in time on different streams of one GPU race - keep them on
+ * one stream, or order the streams.  The kernels leave the counters at zero for the next call. */
+TRN_API trn_status trn_q4k_gemm_noalloc(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 
 /* The legacy 18-byte-block "simplified" Q4_K GEMM, kernel name q4k_gemm_fused: W is n rows x (k/32) blocks
  * (f16 scale + 16 bytes of nibbles, w = scale * q), k a multiple of 32, C as above.  Replaces

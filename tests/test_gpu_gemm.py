@@ -32,8 +32,9 @@ def test_gemm_config_shape_w_14336x4096(gpu, m):
     assert kq.rel_l2(c, _c64("q4k", buf, a, n, k)) <= TOL
 
 
-def test_gemm_config_shape_w_4096x14336(gpu):
-    n, k, m = 4096, 14336, 16
+@pytest.mark.parametrize("m", (1, 4, 16, 64))
+def test_gemm_config_shape_w_4096x14336(gpu, m):
+    n, k = 4096, 14336
     buf, a = kq.gen_matrix("q4k", 1235, n, k), kq.gen_x(4322, m, k)
     c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
     assert kq.rel_l2(c, _c64("q4k", buf, a, n, k)) <= TOL

@@ -37,6 +37,10 @@ asm(".section .rodata\n"
 extern "C" const unsigned char trn_builtin_hsaco_begin[];
 extern "C" const unsigned char trn_builtin_hsaco_end[];
 
+// trn_noalloc.hip: the library's static device scratch buffer (one copy per GPU)
+extern "C" hipError_t trn_noalloc_scratch_setup(int dev);
+extern "C" uint64_t trn_noalloc_scratch(int dev, size_t* bytes);
+
 namespace {
 
 enum Fmt { Q4K = 0, Q5K = 1, Q6K = 2, NFMT = 3 };
@@ -160,6 +164,12 @@ hipError_t device_kernels(DeviceKernels** out) {
     int occ = 0;
     if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&occ, t.gemv_group, 256, 4096 * 4 + 1024) == hipSuccess && occ >= 1)
       t.resident_small = uint32_t(std::min(occ, 4));
+    // this GPU's copy of the static scratch buffer (trn_q4k_gemm_noalloc): found here, once, so that the entry point
+    // itself never has to set anything up
+    if ((e = trn_noalloc_scratch_setup(dev)) != hipSuccess) {
+      (void)hipModuleUnload(m);
+      return e;
+    }
     t.loaded = true;
     d = t;
   }
@@ -791,7 +801,11 @@ trn_status trn_primary_ctx_release(trn_device device) {
 
 trn_status trn_ctx_set_current(trn_ctx ctx) {
   if (!ctx) return TRN_ERROR_INVALID_VALUE;
-  return st(hipSetDevice(ctx->device));
+  TRN_TRY(hipSetDevice(ctx->device));
+  // first use of the device: load the kernels and find this GPU's static scratch buffer now, so that no launcher has
+  // to (one of them promises to allocate nothing)
+  DeviceKernels* d = nullptr;
+  return st(device_kernels(&d));
 }
 
 trn_status trn_ctx_synchronize(void) {
@@ -1293,6 +1307,28 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   return TRN_SUCCESS;
 }
 
+// The Q4_K GEMM for callers that cannot allocate.  Same dispatch as trn_q4k_gemm; the matrix-core form's partial
+// results and counters live in this GPU's copy of the library's static scratch buffer.  After the first use of the
+// library on the device (which loads the kernels and finds the buffer) this calls nothing that allocates or frees.
+trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
+  if (k % 256u != 0) return TRN_ERROR_INVALID_VALUE;
+  if (n == 0 || m == 0) return TRN_SUCCESS;
+  if ((a == 0 && k != 0) || c == 0 || (b == 0 && k != 0)) return TRN_ERROR_INVALID_VALUE;
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  if (!q4k_gemm_f16_ok(a, b, c, m, n, k)) return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));  // no scratch at all
+  DeviceKernels* d = nullptr;
+  TRN_TRY(device_kernels(&d));
+  int dev = 0;
+  TRN_TRY(hipGetDevice(&dev));
+  size_t cap = 0;
+  const uint64_t base = trn_noalloc_scratch(dev, &cap);
+  if (!base) return TRN_ERROR_INVALID_VALUE;
+  // launch_q4k_gemm_f16 answers hipErrorInvalidValue when the product needs more than `cap`: name that case
+  const hipError_t e = launch_q4k_gemm_f16(d, stream, a, b, c, m, n, k, base, cap);
+  if (e == hipErrorInvalidValue) return TRN_ERROR_SCRATCH_TOO_SMALL;
+  return st(e);
+}
+
 // ---- 9. dequantise test surface ----------------------------------------------------------
 trn_status trn_q4k_dequant_f32(trn_stream s, trn_dptr out, trn_dptr w, uint64_t n_sb, int policy) {
   return st(launch_dequant(Q4K, static_cast<hipStream_t>(s), out, w, n_sb, policy));
@@ -1351,9 +1387,11 @@ trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t
 
 const char* trn_error_name(trn_status status) {
   if (status == TRN_ERROR_WAIT_ABANDONED) return "TRN_ERROR_WAIT_ABANDONED";
+  if (status == TRN_ERROR_SCRATCH_TOO_SMALL) return "TRN_ERROR_SCRATCH_TOO_SMALL";
   return hipGetErrorName(static_cast<hipError_t>(status));
 }
 const char* trn_error_string(trn_status status) {
+  if (status == TRN_ERROR_SCRATCH_TOO_SMALL) return "TRN_ERROR_SCRATCH_TOO_SMALL: the product needs more than the library's static scratch buffer";
   if (status == TRN_ERROR_WAIT_ABANDONED) return "TRN_ERROR_WAIT_ABANDONED: a device-side wait of the resident list executor gave up";
   return hipGetErrorString(static_cast<hipError_t>(status));
 }
