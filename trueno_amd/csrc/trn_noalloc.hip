@@ -16,7 +16,9 @@ constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {};
 }  // namespace
 
-static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
+// No `used` attribute here: clang gives a static device variable that host code names an external symbol in the code
+// object, which is how hipGetSymbolAddress finds it; marked `used` it stays a local symbol and the lookup fails.
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 // Once per device, with that device current (the caller serialises): find this GPU's copy and put the counters at
 // zero.  Set-up may allocate and synchronise; the entry point that uses the buffer afterwards does neither.
