@@ -115,14 +115,15 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
 // One entry on this workgroup's share of rows.  Returns false if the barrier wait gave up.
 //   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][k/256 group sums of squares]
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
+// block_threads: blockDim.x, handed in by the kernel (an implicit kernel argument, i.e. a load: the kernel decides when).
 template <int FMT, int U, bool COHERENT = false>
 __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
-                                           f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks) {
+                                           f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks, u32 block_threads) {
   using Q = Quarter<FMT>;
   // The engine is built for whole waves: a block that is not a positive multiple of 64 threads (the reference's own
   // geometry is 32) would divide by zero below and never leave the staging loop.  Uniform exit before any barrier.
-  if (blockDim.x < 64u || (blockDim.x & 63u) != 0u) return true;
-  const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
+  if (block_threads < 64u || (block_threads & 63u) != 0u) return true;
+  const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = block_threads >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;
   const u32 sw_count = slabs < waves ? slabs : waves;
@@ -276,7 +277,7 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
     }
   }
   __syncthreads();
-  for (u32 t = tid; t < rows_per_block; t += blockDim.x) {
+  for (u32 t = tid; t < rows_per_block; t += block_threads) {
     const u32 row = row0 + t;
     if (row < n_dim) {
       float s = part[t];
@@ -319,7 +320,7 @@ __device__ __forceinline__ u32 phases_run(u32 p, const ChainEntry* __restrict__ 
     const PhaseAssign a = assign[static_cast<size_t>(p) * gridDim.x + blockIdx.x];
     if (a.fmt != static_cast<u32>(FMT)) break;
     const ChainEntry e = entries[a.entry];
-    if (!chain_step<FMT, U, true>(e, p ? counters + p * stride : nullptr, spin_limit, status, lds4, s_flag, a.block_id, a.num_blocks))
+    if (!chain_step<FMT, U, true>(e, p ? counters + p * stride : nullptr, spin_limit, status, lds4, s_flag, a.block_id, a.num_blocks, blockDim.x))
       return 0xFFFFFFFFu;
     if (p + 1 < phases) chain_arrive(counters + (p + 1) * stride);
     else __syncthreads();

@@ -69,14 +69,14 @@ __device__ __forceinline__ void gemv_generic_body(float* __restrict__ y, const u
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, 0u, w, x, y};                                               \
-    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
+    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x, blockDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(768)                                                      \
       fmtname##_gemv_flags(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) {\
     extern __shared__ f32x4 lds4[];                                                                      \
     __shared__ u32 s_flag;                                                                               \
     const ChainEntry e = {FMT, k_dim, n_dim, flags, w, x, y};                                            \
-    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                          \
+    chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x, blockDim.x);                                          \
   }                                                                                                      \
   extern "C" __global__ void __launch_bounds__(256)                                                      \
       fmtname##_gemv_generic(float* y, const uint8_t* w, const float* x, u32 k_dim, u32 n_dim, u32 flags) { \
@@ -90,21 +90,48 @@ KQ_GEMV_KERNELS(q6k, FMT_Q6K)
 // Up to eight GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
 // up) in one launch: consecutive runs of workgroups belong to consecutive entries.  Each entry is computed
 // exactly as its own launch would compute it.
-struct GemvGroup {
-  ChainEntry e[8];
-  u32 first[9];      // first[i] .. first[i+1]-1 are the workgroups of entry i
-  u32 count;
+// A workgroup can ask for its first rows only once it knows its matrix, and kernel arguments come from memory: finding
+// the entry through a table in the argument and then reading the entry would be two memory round trips in a row.  The
+// table therefore travels as eight leading scalar arguments, which the build asks the hardware to place in scalar
+// registers when a wave starts (kernel-argument preload); the entry is then one indexed read, whose `hot` part is all
+// that the first loads need.
+struct GemvGroupHot {
+  const uint8_t* w;
+  const float* x;
+  u32 k, n, fmt, flags;
 };
-extern "C" __global__ void __launch_bounds__(768) kq_gemv_group(const GemvGroup g) {
+struct GemvGroupCold {
+  float* y;
+  const float* gamma;
+  const float* x2;
+  const float* residual;
+  float eps;
+  u32 pad;
+};
+struct GemvGroup {
+  GemvGroupHot hot[8];
+  GemvGroupCold cold[8];
+};
+// first1 .. first8: first[j] is the first workgroup of entry j (first[0] = 0; entries that do not exist repeat the grid size)
+extern "C" __global__ void __launch_bounds__(768)
+kq_gemv_group(u32 first1, u32 first2, u32 first3, u32 first4, u32 first5, u32 first6, u32 first7, u32 first8, const GemvGroup g) {
   extern __shared__ f32x4 lds4[];
   __shared__ u32 s_flag;
-  u32 i = 0;
-  while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) ++i;
-  const ChainEntry e = g.e[i];
-  const u32 block_id = blockIdx.x - g.first[i], num_blocks = g.first[i + 1] - g.first[i];
-  if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
-  else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
-  else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks);
+  const u32 fr[9] = {0u, first1, first2, first3, first4, first5, first6, first7, first8};
+  u32 i = 0, wg0 = fr[0], wg1 = fr[1];
+#pragma unroll
+  for (u32 j = 1; j < 8; ++j)
+    if (blockIdx.x >= fr[j]) { i = j; wg0 = fr[j]; wg1 = fr[j + 1]; }       // first[] never decreases
+  GemvGroupHot h = g.hot[i];
+  const GemvGroupCold c = g.cold[i];
+  // the block size is an implicit kernel argument, a load like the entry's: all of them in flight together, one wait
+  u32 block_threads = blockDim.x;
+  asm volatile("" : "+s"(block_threads), "+s"(h.k), "+s"(h.flags));
+  const ChainEntry e = {h.fmt, h.k, h.n, h.flags, h.w, h.x, c.y, c.gamma, c.x2, c.residual, c.eps, 0u};
+  const u32 block_id = blockIdx.x - wg0, num_blocks = wg1 - wg0;
+  if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
+  else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
+  else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
 }
 
 // The list as phases of independent entries in one resident launch, one workgroup of 12 waves per CU.
@@ -221,7 +248,7 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
     for (u32 r = blockIdx.y; r < m; r += gridDim.y) {                                                    \
       const ChainEntry e = {FMT, k, n, 0u, b_quant, a + static_cast<size_t>(r) * k,                      \
                             c + static_cast<size_t>(r) * n};                                             \
-      chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x);                                        \
+      chain_step<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, blockIdx.x, gridDim.x, blockDim.x);                                        \
       __syncthreads();                                                                                   \
     }                                                                                                    \
   }                                                                                                      \

@@ -89,6 +89,8 @@ std::atomic<int> g_tune_row_groups{0};
 std::atomic<int> g_tune_batch_mode{0};   // 0: launches (default); 1: resident phases + barriers
 std::atomic<int> g_tune_chain_spin_limit{0};
 std::atomic<int> g_tune_group_off{0};
+std::atomic<int> g_tune_group_pool_off{0};
+std::atomic<int> g_tune_group_pool_waves{0};  // 1: grouped launches cut every entry's rows evenly (no run-time pools)
 std::atomic<int> g_tune_gemm_mfma_off{0};   // 1: the Q4_K GEMM never takes the matrix-core form
 std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 std::atomic<int> g_tune_attention_min_steps{0};
@@ -1155,12 +1157,11 @@ trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
 }
 
 namespace {
-struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip
-  ChainEntryHost e[kGroupMax];
-  uint32_t first[kGroupMax + 1];
-  uint32_t count;
+struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip: what a workgroup's first loads need, then the rest
+  struct Hot { uint64_t w, x; uint32_t k, n, fmt, flags; } hot[kGroupMax];
+  struct Cold { uint64_t y, gamma, x2, residual; float eps; uint32_t pad; } cold[kGroupMax];
 };
-static_assert(sizeof(GemvGroupHost) == kGroupMax * 72 + (kGroupMax + 1) * 4 + 4, "GemvGroup layout");
+static_assert(sizeof(GemvGroupHost) == kGroupMax * (32 + 40), "GemvGroup layout");
 
 bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
@@ -1190,30 +1191,31 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::max(1u, 12u / waves);
   const double target = double(d->cu_count) * per_cu;
   GemvGroupHost g{};
+  uint32_t first[kGroupMax + 1] = {};
   uint32_t lds = 0;
-  g.first[0] = 0;
   for (uint32_t i = 0; i < len; ++i) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves), groups = waves / sw;
+    const double bytes = cost_of(e);
+    const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
+    const uint64_t x_bytes = uint64_t(e.k) * 4u;
+    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags};
+    g.cold[i] = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
     // workgroups of 8 waves or more hand their row batches out among the waves: a share need not be a whole
     // number of rounds of all waves
     const uint32_t ug = waves >= 8u ? kGemvRowsPerBatch : kGemvRowsPerBatch * groups;
-    const double bytes = cost_of(e);
-    const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
     uint64_t rows = (uint64_t(e.n) + share - 1) / share;
     rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
-    const uint64_t x_bytes = uint64_t(e.k) * 4u;
     if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return hipErrorInvalidValue;
     const uint64_t max_rows = (kFastLdsLimit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
     rows = std::min<uint64_t>(rows, max_rows);
     const uint32_t grid = uint32_t((uint64_t(e.n) + rows - 1) / rows);
     lds = std::max<uint32_t>(lds, uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch));
-    g.e[i] = entry_of(e);
-    g.first[i + 1] = g.first[i] + grid;
+    first[i + 1] = first[i] + grid;
   }
-  g.count = len;
-  void* args[] = {&g};
-  return hipModuleLaunchKernel(d->gemv_group, g.first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
+  for (uint32_t i = len; i < kGroupMax; ++i) first[i + 1] = first[len];   // entries that do not exist own no workgroup
+  void* args[] = {&first[1], &first[2], &first[3], &first[4], &first[5], &first[6], &first[7], &first[8], &g};
+  return hipModuleLaunchKernel(d->gemv_group, first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
 }
 }  // namespace
 
