@@ -6,15 +6,20 @@ A step is one 7B-style decode weight pass: 32 layers x {Q,K,V,O: Q4_K 4096x4096;
 distinct, seeded synthetic weights resident in HBM (far beyond the 256 MB Infinity Cache, so every
 pass streams from HBM).  Data flow, per layer: a fresh x_l ~ N(0,1) feeds q, k, v, gate and up; o
 consumes the RMS-normalised output of q; down consumes the RMS-normalised output of gate; the head
-consumes the RMS-normalised output of the last down.  The list goes to the library in one call, in
-layer order (trn_kquant_gemv_batch).  `value` is algorithmic bytes (weights + x + y, each once)
-over wall time.  The same 225 GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h;
-o <- q; gate,up <- o; down <- gate; h <- down) are timed too and reported in `extra`.
+consumes the RMS-normalised output of the last down.  The list (trueno_amd.decode_pass, the one the
+GPU parity test checks) goes to the library in one call, in layer order (trn_kquant_gemv_batch).
+`value` is algorithmic bytes (weights + x + y, each once) over wall time.  After the timed region the
+last layer's outputs and the logits are checked against fp64 on their actual inputs.  The same 225
+GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate;
+h <- down) are timed too: `strict_decoder_chain` in `config`.
 
-Prints one JSON line.  Extra fields: `roofline` for the dominant kernel (kq_gemv_group: the launches that carry
-up to four independent neighbouring entries, 64 per pass, 3.99 of the 4.13 GB), its launches of one pass timed
-with HIP events on their stream; `cpu_baseline`: the CPU port
-(oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.
+Prints one JSON line.  `roofline`: the dominant kernel (kq_gemv_group: the launches that carry several
+independent entries, 64 per pass, 3.99 of the 4.13 GB), its launches of one pass timed with HIP events on
+their stream, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
+(oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other
+benchmark configurations, timed as launches back to back over at least 1 GiB of distinct copies
+(200 launches, median of 5 batches), one copy over and over ("hot": from the last-level cache), and
+eight independent copies per library call (the grouped launch in steady state).
 """
 import argparse
 import ctypes as C
@@ -29,20 +34,11 @@ sys.path.insert(0, ROOT)
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per kq_gemv_group launch, averaged over the 64 such launches of the full pass: rocprofv3
-# FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the counter reads for kq_copy_u128 on
-# 256 MiB (profiles/kquant_gemv_hbm_traffic_pmc.md).  Counters cannot be read from inside this
-# process, so the figure is carried here and re-measured whenever the kernel changes.
-GROUP_TRAFFIC_BYTES_PER_LAUNCH = 63_595_450
-LAYERS = 32
-SB = {"q4k": 144, "q5k": 176, "q6k": 210}
-LAYER_MATS = [("q", "q4k", 4096, 4096), ("k", "q4k", 4096, 4096), ("v", "q4k", 4096, 4096), ("o", "q4k", 4096, 4096),
-              ("gate", "q4k", 11008, 4096), ("up", "q4k", 11008, 4096), ("down", "q6k", 4096, 11008)]
-HEAD = ("head", "q6k", 32000, 4096)
-
-
-def alg_bytes(fmt, n, k):
-    return n * (k // 256) * SB[fmt] + 4 * k + 4 * n
+TOL = 1e-5                      # relative L2 against fp64, as in the parity tests
+GIB = 1 << 30
+# HBM bytes per kq_gemv_group launch as the hardware counters saw them: written next to the rocprofv3 summaries by
+# the script that makes them (python -m trueno_amd.rocprof_summary), with the commit it was measured at.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "kquant_gemv_group_traffic.json")
 
 
 def main() -> int:
@@ -51,10 +47,14 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-configs", action="store_true", help="skip the single-launch table of configurations 1, 2, 3 and 5")
-    ap.add_argument("--no-executors", action="store_true", help="skip the comparison runs of the opt-in one-launch executors")
-    ap.add_argument("--layers", type=int, default=LAYERS, help=argparse.SUPPRESS)
+    ap.add_argument("--no-configs", action="store_true", help="skip the tables of configurations 1, 2, 3 and 5 and of the path's neighbours")
+    ap.add_argument("--no-executors", action="store_true", help="skip the comparison run of the opt-in one-launch executor")
+    ap.add_argument("--pass-only", action="store_true",
+                    help="only the timed passes and the launches of the roofline figure (for counter runs: every dispatch of the "
+                         "dominant kernel then belongs to the pass)")
     args = ap.parse_args()
+    if args.pass_only:
+        args.no_cpu_baseline = args.no_configs = args.no_executors = True
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus must be 1 (several GPUs would each take a range of rows of "
               "every matrix and exchange the output vectors)", file=sys.stderr)
@@ -63,16 +63,16 @@ def main() -> int:
     import trueno_amd as t
     from oracle import kquant as kq
     from trueno_amd import _ffi
+    from trueno_amd.decode_pass import HEAD, LAYER_MATS, SB, DecodePass, alg_bytes
 
     L = _ffi.lib()
     ctx = t.CudaContext(0)
     stream = t.CudaStream(ctx)
-    layers = args.layers
+    layers = 32
 
     # ---- seeded synthetic weights, distinct per layer, resident in HBM before timing -------------
     t_gen = time.time()
-    weights, xs = [], []
-    host_layer0 = {}
+    weights, xs, host_layer0, host_last = [], [], {}, {}
     for layer in range(layers):
         mats = {}
         for mi, (name, fmt, n, k) in enumerate(LAYER_MATS):
@@ -80,75 +80,28 @@ def main() -> int:
             mats[name] = t.GpuBuffer.from_host(ctx, host)
             if layer == 0:
                 host_layer0[name] = host
+            if layer == layers - 1:
+                host_last[name] = host
         weights.append(mats)
-        xs.append((t.GpuBuffer.from_host(ctx, kq.gen_x(4321 + layer, 4096)),
-                   t.GpuBuffer.from_host(ctx, kq.gen_x(8321 + layer, 11008))))
-    head_w = t.GpuBuffer.from_host(ctx, kq.gen_matrix(HEAD[1], 999, HEAD[2], HEAD[3]))
-    y = {n: t.GpuBuffer(ctx, n, np.float32) for n in (4096, 11008, 32000)}
-    ys = {name: t.GpuBuffer(ctx, n, np.float32) for name, _, n, _ in LAYER_MATS}
+        xs.append(kq.gen_x(4321 + layer, 4096))
+    host_head = kq.gen_matrix(HEAD[1], 999, HEAD[2], HEAD[3])
+    dp = DecodePass(ctx, weights, t.GpuBuffer.from_host(ctx, host_head), [t.GpuBuffer.from_host(ctx, x) for x in xs])
+    x11008 = t.GpuBuffer.from_host(ctx, kq.gen_x(8321, 11008))
+    y = {n: t.GpuBuffer(ctx, n, np.float32) for n in (4096, 11008, 14336, 32000)}
     print(f"[bench] generated and uploaded {layers} layers in {time.time() - t_gen:.1f} s", file=sys.stderr, flush=True)
 
-    # ---- the pass as one list, in layer order.  Data flow per layer: a fresh x_l ~ N(0,1) feeds q, k, v, gate and
-    #      up; o consumes the RMS-normalised output of q; down consumes the RMS-normalised output of gate; the head
-    #      consumes the RMS-normalised output of the last down.  The library works out from the pointers which
-    #      neighbouring entries are independent of one another.
+    batch, strict_batch, layer_batch = dp.build("fresh_x"), dp.build("strict"), dp.build("folded")
+    entry_bytes, entry_names = dp.entry_bytes(), dp.entry_names()
+    total_bytes, weight_bytes = sum(entry_bytes), dp.weight_bytes()
+    act, logits, head_w = dp.act, dp.logits, dp.head_w
     NORM = t.GemvBatch.NORM_INPUT
-    act = {nm: t.GpuBuffer(ctx, n, np.float32) for nm, n in (("q", 4096), ("k", 4096), ("v", 4096), ("o", 4096),
-                                                             ("gate", 11008), ("up", 11008), ("down", 4096))}
-    logits = y[32000]
-    src_of = {"q": None, "k": None, "v": None, "o": "q", "gate": None, "up": None, "down": "gate"}
-
-    def build_pass(strict):
-        """strict: the serial data flow of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate; h <- down)."""
-        b = t.GemvBatch()
-        nbytes = wbytes = 0
-        h = xs[0][0]
-        for layer in range(layers):
-            for name, fmt, n, k in LAYER_MATS:
-                if strict:
-                    src = {"q": None, "k": None, "v": None, "o": "q", "gate": "o", "up": "o", "down": "gate"}[name]
-                    x, flags = (h if src is None else act[src]), NORM
-                else:
-                    src = src_of[name]
-                    x, flags = (xs[layer][0], 0) if src is None else (act[src], NORM)
-                b.add(fmt, k, n, act[name], weights[layer][name], x, flags)
-                nbytes += alg_bytes(fmt, n, k)
-                wbytes += n * (k // 256) * SB[fmt]
-            h = act["down"]
-        b.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, act["down"], NORM)
-        nbytes += alg_bytes(HEAD[1], HEAD[2], HEAD[3])
-        wbytes += HEAD[2] * (HEAD[3] // 256) * SB[HEAD[1]]
-        return b, nbytes, wbytes
-
-    for kv in filter(None, os.environ.get("TRN_BENCH_TUNE", "").split(",")):      # working aid: library tuning keys
-        key, val = kv.split("=")
-        assert L.trn_set_tuning(key.encode(), int(val)) == 0, kv
-    def build_layer_pass():
-        """the decoder's serial data flow with the element-wise steps of a layer folded into the entries: q,k,v <-
-        rmsnorm(h)*g1; h1 = h + o(q); gate,up <- rmsnorm(h1)*g2; h = h1 + down(silu(gate)*up); head <- rmsnorm(h)*g"""
-        b = t.GemvBatch()
-        res = [t.GpuBuffer.from_host(ctx, kq.gen_x(777, 4096)), t.GpuBuffer(ctx, 4096, np.float32)]   # h, h1
-        gammas = [t.GpuBuffer.from_host(ctx, np.abs(kq.gen_x(780 + i, 4096)) + np.float32(0.5)) for i in range(2)]
-        w_of = lambda layer, name: weights[layer][name]
-        for layer in range(layers):
-            for name in ("q", "k", "v"):
-                b.add("q4k", 4096, 4096, act[name], w_of(layer, name), res[0], NORM, gamma=gammas[0], norm_eps=1e-5)
-            b.add("q4k", 4096, 4096, res[1], w_of(layer, "o"), act["q"], 0, residual=res[0])
-            for name in ("gate", "up"):
-                b.add("q4k", 4096, 11008, act[name], w_of(layer, name), res[1], NORM, gamma=gammas[1], norm_eps=1e-5)
-            b.add("q6k", 11008, 4096, res[0], w_of(layer, "down"), act["gate"], 0, x2=act["up"], residual=res[1])
-        b.add(HEAD[1], HEAD[3], HEAD[2], logits, head_w, res[0], NORM, gamma=gammas[0], norm_eps=1e-5)
-        b.keep = (res, gammas)
-        return b
-
-    batch, total_bytes, weight_bytes = build_pass(False)
-    strict_batch, _, _ = build_pass(True)
-    layer_batch = build_layer_pass()
 
     def ev():
         e = C.c_void_p()
         assert L.trn_event_create(C.byref(e)) == 0
         return e
+
+    e0, e1 = ev(), ev()
 
     # one plain copy of known size (256 MiB read + 256 MiB written): the yardstick that profiler byte
     # counters of the same run are scaled by
@@ -168,7 +121,6 @@ def main() -> int:
         for _ in range(warmup):
             batch.launch(stream)
         stream.synchronize()
-        e0, e1 = ev(), ev()
         t0 = time.perf_counter()
         L.trn_event_record(e0, stream.raw())
         for _ in range(steps):
@@ -178,29 +130,45 @@ def main() -> int:
         wall = (time.perf_counter() - t0) * 1e3
         return wall / steps, elapsed_ms(e0, e1) / steps
 
-    # ---- timed region: W warm-up passes, then exactly K passes (one cooperative launch per pass) ----
+    # ---- timed region: W warm-up passes, then exactly K passes ------------------------------------------------
     ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
-    assert np.all(np.isfinite(logits.copy_to_host())), "the pass produced non-finite logits"
+
+    # ---- what the timed passes left behind, against fp64 on the actual inputs: the last layer (whose outputs are still
+    #      in the shared activation buffers) and the logits ----------------------------------------------------------
+    def norm64(v, eps=1e-6):
+        v = v.astype(np.float64)
+        return v / np.sqrt(np.mean(v * v) + eps)
+
+    got = {nm: b.copy_to_host() for nm, b in act.items()}
+    got["logits"] = logits.copy_to_host()
+    x_last = xs[layers - 1].astype(np.float64)
+    inputs = {"q": x_last, "k": x_last, "v": x_last, "gate": x_last, "up": x_last, "o": norm64(got["q"]), "down": norm64(got["gate"])}
+    verification = {}
+    for name, fmt, n, k in LAYER_MATS:
+        w = kq.dequant_matrix(fmt, host_last[name], n, k)
+        verification[f"layer{layers - 1}_{name}"] = float(kq.rel_l2(got[name], w @ inputs[name]))
+        del w
+    verification["head"] = float(kq.rel_l2(got["logits"], kq.dequant_matrix(HEAD[1], host_head, HEAD[2], HEAD[3]) @ norm64(got["down"])))
+    worst = max(verification.values())
+    assert np.all(np.isfinite(got["logits"])) and worst <= TOL, f"the timed pass is wrong: {verification}"
+    del host_last, host_head
 
     # ---- dominant kernel: kq_gemv_group.  The library puts entries that are independent of one another (and of what
     #      they would overtake) into one launch of this kernel; trn_kquant_gemv_plan says which entry of the pass goes
-    #      into which launch.  The launches of the pass that hold two or more entries (all of it but a few single
-    #      GEMVs, which take the single-GEMV kernels) are issued here one list each, in pass order, back to back on
-    #      the stream, bracketed by HIP events on that stream.
+    #      into which launch.  The launches of the pass that hold two or more entries (all of it but the head, which
+    #      takes the single-GEMV kernel) are issued here one list each, in pass order, back to back on the stream,
+    #      bracketed by HIP events on that stream.
     launch_of = batch.plan()
     members = {}
     for i, l in enumerate(launch_of):
         members.setdefault(l, []).append(i)
-    entry_bytes = [alg_bytes(fmt, n, k) for _ in range(layers) for _, fmt, n, k in LAYER_MATS] + [alg_bytes(HEAD[1], HEAD[2], HEAD[3])]
-    entry_names = [name for _ in range(layers) for name, _, _, _ in LAYER_MATS] + ["head"]
     kinds = {}
     for l in sorted(members):
         sig = "[" + ",".join(entry_names[i] for i in members[l]) + "]"
         kinds[sig] = kinds.get(sig, 0) + 1
     print("[bench] launches of the pass: " + ", ".join(f"{c} x {sig}" for sig, c in kinds.items()), file=sys.stderr, flush=True)
-    groups = []
-    grp_bytes = 0
+    groups, grp_bytes = [], 0
     for l in sorted(members):
         if len(members[l]) >= 2:
             g = batch.subset(members[l])
@@ -208,7 +176,6 @@ def main() -> int:
             groups.append(g)
             grp_bytes += sum(entry_bytes[i] for i in members[l])
     n_grp = len(groups)
-    e0, e1 = ev(), ev()
     grp_ms = []
     for _ in range(5):
         for g in groups:
@@ -224,111 +191,142 @@ def main() -> int:
     grp_bytes_per_launch = grp_bytes / n_grp
     achieved = grp_bytes_per_launch / (grp_ms * 1e-3) / 1e9
 
-    # ---- the same GEMVs wired as the strictly serial chain of a decoder ------------------------------------
-    strict_ms, _ = run_passes(max(3, args.steps // 2), 2, strict_batch)
-    layer_ms, _ = run_passes(max(3, args.steps // 2), 2, layer_batch)
-
-    # ---- the same list through the one-launch executors (opt-in), for comparison ------------------------
-    other_modes = {}
-    for mode, label in (() if args.no_executors else ((1, "resident_phases"),)):
-        L.trn_set_tuning(b"batch_mode", mode)
-        ms, _ = run_passes(max(3, args.steps // 2), 1)
-        other_modes[label] = round(ms * 1e3, 1)
-    L.trn_set_tuning(b"batch_mode", 0)
-
-    # ---- per-shape single-launch table (cold: rotates through the layers' copies) -----------------------
-    shapes = {}
-    for name, fmt, n, k in LAYER_MATS[3:] + [HEAD]:
-        b = t.GemvBatch()
-        reps = layers if name != "head" else 8
-        for r in range(reps):
-            wbuf = head_w if name == "head" else weights[r % layers][name]
-            b.add(fmt, k, n, y[n], wbuf, xs[r % layers][1 if k == 11008 else 0])
-        b.launch(stream)
-        stream.synchronize()
+    # a bare read of as many bytes per launch, nothing computed, launches back to back over cold data: what the
+    # memory system and a kernel launch allow for a launch of this size
+    read_bytes = int(grp_bytes_per_launch) // 16 * 16
+    pieces = GIB // read_bytes
+    read_src = t.GpuBuffer(ctx, GIB // 4, np.float32)
+    read_us = []
+    for _ in range(5):
         L.trn_event_record(e0, stream.raw())
-        b.launch(stream)
+        for r in range(64):
+            L.trn_read_u128(stream.raw(), read_src.as_ptr() + (r % pieces) * read_bytes, read_bytes, y[4096].as_ptr())
         L.trn_event_record(e1, stream.raw())
         stream.synchronize()
-        us = elapsed_ms(e0, e1) * 1e3 / reps
-        key = f"{fmt}_{n}x{k}" + ("_hot" if name == "head" else "")
-        shapes[key] = {"us": round(us, 2), "gbps": round(alg_bytes(fmt, n, k) / us / 1e3, 1),
-                       "frac_of_peak": round(alg_bytes(fmt, n, k) / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        read_us.append(elapsed_ms(e0, e1) * 1e3 / 64)
+    read_us = sorted(read_us)[2]
+    read_src.free()
 
-    # ---- the other benchmark configurations, one launch each, cold (16 distinct device copies in rotation) --------
-    configs = {}
-    if not args.no_configs:
-        def timed(launch, reps):
-            for r in range(reps):
-                launch(r)
-            stream.synchronize()
+    traffic = None
+    if os.path.exists(TRAFFIC_JSON):
+        with open(TRAFFIC_JSON) as f:
+            traffic = json.load(f)
+
+    # ---- the same GEMVs wired as the strictly serial chain of a decoder ------------------------------------
+    strict_ms = layer_ms = None
+    if not args.pass_only:
+        strict_ms, _ = run_passes(max(3, args.steps // 2), 2, strict_batch)
+        layer_ms, _ = run_passes(max(3, args.steps // 2), 2, layer_batch)
+
+    # ---- the same list through the one-launch executor (opt-in), for comparison ------------------------
+    other_modes = {}
+    if not args.no_executors:
+        L.trn_set_tuning(b"batch_mode", 1)
+        ms, _ = run_passes(max(3, args.steps // 2), 1)
+        other_modes["resident_phases"] = round(ms * 1e3, 1)
+        L.trn_set_tuning(b"batch_mode", 0)
+
+    # ---- timing protocol of the other configurations: launches back to back on the stream, no host wait inside;
+    #      20 to warm up, then 5 batches of 200, the median batch counts.  "cold": every launch another of enough
+    #      distinct device copies to make 1 GiB (nothing comes from the 256 MB last-level cache); "hot": one copy over
+    #      and over; "grouped": eight copies per library call, which the library issues as one launch.
+    def protocol(launch, reps=200, warm=20, batches=5):
+        for r in range(warm):
+            launch(r)
+        stream.synchronize()
+        us, enq = [], []
+        for _ in range(batches):
+            t0 = time.perf_counter()
             L.trn_event_record(e0, stream.raw())
             for r in range(reps):
                 launch(r)
             L.trn_event_record(e1, stream.raw())
+            enq.append((time.perf_counter() - t0) * 1e6 / reps)
             stream.synchronize()
-            return elapsed_ms(e0, e1) * 1e3 / reps
+            us.append(elapsed_ms(e0, e1) * 1e3 / reps)
+        return sorted(us)[batches // 2], sorted(enq)[batches // 2]
 
-        copies = 16
+    def copies_of(host, nbytes):
+        n = max(2, -(-GIB // nbytes))
+        first = t.GpuBuffer.from_host(ctx, host)
+        bufs = [first]
+        for _ in range(n - 1):
+            b = t.GpuBuffer(ctx, first.len(), np.uint8)
+            b.copy_from_buffer(first)
+            bufs.append(b)
+        return bufs
+
+    def rate(nbytes, us):
+        return {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1), "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+    configs = {}
+    if not args.no_configs:
         for label, fmt, n, k in (("1_q4k_gemv", "q4k", 4096, 4096), ("2_q6k_gemv", "q6k", 4096, 4096),
                                  ("2_q6k_gemv", "q6k", 32000, 4096), ("3_q5k_gemv", "q5k", 11008, 4096),
-                                 ("3_q5k_gemv", "q5k", 4096, 11008)):
-            host = kq.gen_matrix(fmt, 1234, n, k)
-            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
-            xb = xs[0][1 if k == 11008 else 0]
+                                 ("3_q5k_gemv", "q5k", 4096, 11008), ("4_q4k_gemv", "q4k", 11008, 4096),
+                                 ("4_q6k_gemv", "q6k", 4096, 11008)):
+            nbytes = alg_bytes(fmt, n, k)
+            bufs = copies_of(kq.gen_matrix(fmt, 1234, n, k), nbytes)
+            nc = len(bufs)
+            xb = x11008 if k == 11008 else dp.xs[0]
             fn = getattr(L, f"trn_{fmt}_gemv")
-            us = timed(lambda r: fn(stream.raw(), y[n].as_ptr(), bufs[r % copies].as_ptr(), xb.as_ptr(), k, n), 2 * copies)
-            # the same launch on one copy over and over: the weights come from the 256 MB last-level cache, not from HBM
-            hot = timed(lambda r: fn(stream.raw(), y[n].as_ptr(), bufs[0].as_ptr(), xb.as_ptr(), k, n), 2 * copies)
-            configs[f"{label}_{n}x{k}"] = {"us": round(us, 2), "gbps": round(alg_bytes(fmt, n, k) / us / 1e3, 1),
-                                            "frac_of_peak": round(alg_bytes(fmt, n, k) / us / 1e3 / HBM_PEAK_GBPS, 4),
-                                            "us_cache_hot": round(hot, 2)}
-            for b in bufs:
+            cold, enq = protocol(lambda r: fn(stream.raw(), y[n].as_ptr(), bufs[r % nc].as_ptr(), xb.as_ptr(), k, n))
+            hot, _ = protocol(lambda r: fn(stream.raw(), y[n].as_ptr(), bufs[0].as_ptr(), xb.as_ptr(), k, n))
+            ys8 = [t.GpuBuffer(ctx, n, np.float32) for _ in range(8)]
+            lists = []
+            for c0 in range(0, nc - nc % 8 if nc >= 8 else nc, 8):
+                b = t.GemvBatch()
+                for j in range(8):
+                    b.add(fmt, k, n, ys8[j], bufs[(c0 + j) % nc], xb)
+                assert len(set(b.plan())) == 1
+                lists.append(b)
+            grouped, _ = protocol(lambda r: lists[r % len(lists)].launch(stream), reps=25, warm=4)
+            row = {"cold": rate(nbytes, cold), "hot_last_level_cache": rate(nbytes, hot),
+                   "grouped_8_per_call_cold": rate(nbytes, grouped / 8), "copies": nc, "host_enqueue_us_per_launch": round(enq, 2)}
+            configs[f"{label}_{n}x{k}"] = row
+            for b in bufs + ys8:
                 b.free()
         for n, k in ((14336, 4096), (4096, 14336)):
-            host = kq.gen_matrix("q4k", 1238, n, k)
-            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            wbytes = n * (k // 256) * 144
+            bufs = copies_of(kq.gen_matrix("q4k", 1238, n, k), wbytes)
+            nc = len(bufs)
             for m in (1, 4, 16, 64):
                 a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
                 c = t.GpuBuffer(ctx, m * n, np.float32)
-                us = timed(lambda r: L.trn_q4k_gemm(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k),
-                           2 * copies)
-                nbytes = n * (k // 256) * 144 + 4 * m * k + 4 * m * n
-                configs[f"5_q4k_gemm_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
-                                                       "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
-                                                       "tflops": round(2.0 * m * n * k / us / 1e6, 1)}
+                cold, enq = protocol(lambda r: L.trn_q4k_gemm(stream.raw(), a.as_ptr(), bufs[r % nc].as_ptr(), c.as_ptr(), m, n, k))
+                hot, _ = protocol(lambda r: L.trn_q4k_gemm(stream.raw(), a.as_ptr(), bufs[0].as_ptr(), c.as_ptr(), m, n, k))
+                nbytes = wbytes + 4 * m * k + 4 * m * n
+                row = {"cold": rate(nbytes, cold), "hot_last_level_cache": rate(nbytes, hot), "tflops": round(2.0 * m * n * k / cold / 1e6, 1),
+                       "copies": nc, "host_enqueue_us_per_launch": round(enq, 2)}
+                configs[f"5_q4k_gemm_{n}x{k}_m{m}"] = row
                 a.free()
                 c.free()
             for b in bufs:
                 b.free()
 
-        # the GEMM entry points outside BASELINE's configurations: Q5_K / Q6_K (VALU engine per row of A) and the
-        # legacy 18-byte format of q4k_gemm_fused, 4096 x 4096, cold
+        # the GEMM entry points outside BASELINE's configurations: Q5_K / Q6_K and the legacy 18-byte format of
+        # q4k_gemm_fused, 4096 x 4096
         n = k = 4096
         for fmt in ("q5k", "q6k"):
-            host = kq.gen_matrix(fmt, 1239, n, k)
-            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+            bufs = copies_of(kq.gen_matrix(fmt, 1239, n, k), n * (k // 256) * SB[fmt])
+            nc = len(bufs)
             fn = getattr(L, f"trn_{fmt}_gemm")
-            for m in (4, 16):
+            for m in (4, 16, 64):
                 a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
                 c = t.GpuBuffer(ctx, m * n, np.float32)
-                us = timed(lambda r: fn(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k), 2 * copies)
-                nbytes = alg_bytes(fmt, n, k) + 4 * (m - 1) * (k + n)
-                configs[f"x_{fmt}_gemm_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
-                                                         "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+                cold, _ = protocol(lambda r: fn(stream.raw(), a.as_ptr(), bufs[r % nc].as_ptr(), c.as_ptr(), m, n, k), reps=100, warm=8)
+                configs[f"x_{fmt}_gemm_{n}x{k}_m{m}"] = {"cold": rate(alg_bytes(fmt, n, k) + 4 * (m - 1) * (k + n), cold), "copies": nc}
                 a.free()
                 c.free()
             for b in bufs:
                 b.free()
-        host = kq.gen_q4k_simplified(np.random.default_rng(1240), n * (k // 32))
-        bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
+        bufs = copies_of(kq.gen_q4k_simplified(np.random.default_rng(1240), n * (k // 32)), n * (k // 32) * 18)
+        nc = len(bufs)
         for m in (1, 4):
             a = t.GpuBuffer.from_host(ctx, kq.gen_x(4321, m, k).reshape(-1))
             c = t.GpuBuffer(ctx, m * n, np.float32)
-            us = timed(lambda r: L.trn_q4k_gemm_fused(stream.raw(), a.as_ptr(), bufs[r % copies].as_ptr(), c.as_ptr(), m, n, k), 2 * copies)
-            nbytes = n * (k // 32) * 18 + 4 * m * (k + n)
-            configs[f"x_q4k_gemm_fused_{n}x{k}_m{m}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
-                                                        "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            cold, _ = protocol(lambda r: L.trn_q4k_gemm_fused(stream.raw(), a.as_ptr(), bufs[r % nc].as_ptr(), c.as_ptr(), m, n, k), reps=100, warm=8)
+            configs[f"x_q4k_gemm_fused_{n}x{k}_m{m}"] = {"cold": rate(n * (k // 32) * 18 + 4 * m * (k + n), cold), "copies": nc}
             a.free()
             c.free()
         for b in bufs:
@@ -339,73 +337,44 @@ def main() -> int:
     if not args.no_configs:
         hid, ffn = 4096, 11008
         g_a, g_b, g_o, g_g = (t.GpuBuffer.from_host(ctx, kq.gen_x(9000 + i, ffn)) for i in range(4))
-        for label, fn in (("residual_add_4096", lambda: L.trn_residual_add(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), hid)),
-                          ("rmsnorm_4096", lambda: L.trn_rmsnorm(stream.raw(), g_a.as_ptr(), g_o.as_ptr(), g_g.as_ptr(), hid, C.c_float(1e-5))),
-                          ("fused_residual_rmsnorm_4096", lambda: L.trn_fused_residual_rmsnorm(
+        for label, fn in (("residual_add_4096", lambda r: L.trn_residual_add(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), hid)),
+                          ("rmsnorm_4096", lambda r: L.trn_rmsnorm(stream.raw(), g_a.as_ptr(), g_o.as_ptr(), g_g.as_ptr(), hid, C.c_float(1e-5))),
+                          ("fused_residual_rmsnorm_4096", lambda r: L.trn_fused_residual_rmsnorm(
                               stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), g_g.as_ptr(), hid, C.c_float(1e-5))),
-                          ("fused_swiglu_11008", lambda: L.trn_fused_swiglu(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), ffn))):
-            for _ in range(8):
-                fn()
-            stream.synchronize()
-            L.trn_event_record(e0, stream.raw())
-            for _ in range(64):
-                fn()
-            L.trn_event_record(e1, stream.raw())
-            stream.synchronize()
-            glue_us[label] = round(elapsed_ms(e0, e1) * 1e3 / 64, 2)
+                          ("fused_swiglu_11008", lambda r: L.trn_fused_swiglu(stream.raw(), g_a.as_ptr(), g_b.as_ptr(), g_o.as_ptr(), ffn))):
+            us, _ = protocol(fn, reps=100, warm=8)
+            glue_us[label] = round(us, 2)
 
-    # ---- the f32 GEMV of gemv.rs (A is K x N row-major), one launch, cold --------------------------------------
+    # ---- the f32 GEMV of gemv.rs (A is K x N row-major) ---------------------------------------------------------
     f32_gemv = {}
     if not args.no_configs:
         rng = np.random.default_rng(55)
-        for k, n, copies in ((4096, 4096, 8), (4096, 11008, 4)):
-            host = rng.standard_normal(k * n, dtype=np.float32)
-            bufs = [t.GpuBuffer.from_host(ctx, host) for _ in range(copies)]
-            xb, yb = xs[0][0], y[n if n in y else 11008]
-            def launch(r):
-                return L.trn_gemv_f32(stream.raw(), yb.as_ptr(), bufs[r % copies].as_ptr(), xb.as_ptr(), k, n)
-            for r in range(copies):
-                launch(r)
-            stream.synchronize()
-            L.trn_event_record(e0, stream.raw())
-            for r in range(2 * copies):
-                launch(r)
-            L.trn_event_record(e1, stream.raw())
-            stream.synchronize()
-            us = elapsed_ms(e0, e1) * 1e3 / (2 * copies)
+        for k, n in ((4096, 4096), (4096, 11008)):
             nbytes = 4 * k * n + 4 * k + 4 * n
-            f32_gemv[f"k{k}_n{n}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
-                                      "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            bufs = copies_of(rng.standard_normal(k * n, dtype=np.float32).view(np.uint8), nbytes)
+            nc = len(bufs)
+            xb, yb = dp.xs[0], y[n]
+            cold, _ = protocol(lambda r: L.trn_gemv_f32(stream.raw(), yb.as_ptr(), bufs[r % nc].as_ptr(), xb.as_ptr(), k, n), reps=100, warm=8)
+            f32_gemv[f"k{k}_n{n}"] = {"cold": rate(nbytes, cold), "copies": nc}
             for b in bufs:
                 b.free()
 
-    # ---- single-query attention over a KV cache of 7B shape (32 heads x 128), one launch, cold ------------------
+    # ---- single-query attention over a KV cache of 7B shape (32 heads x 128) -----------------------------------
     attention = {}
     if not args.no_configs:
         rng = np.random.default_rng(66)
         heads, dim = 32, 128
         for seq in (512, 2048, 8192):
-            copies = 6
-            kvs = [(t.GpuBuffer.from_host(ctx, rng.standard_normal(heads * seq * dim, dtype=np.float32)),
-                    t.GpuBuffer.from_host(ctx, rng.standard_normal(heads * seq * dim, dtype=np.float32))) for _ in range(copies)]
-            qb, ob = xs[0][0], y[4096]
-            def launch(r):
-                return L.trn_incremental_attention(stream.raw(), qb.as_ptr(), kvs[r % copies][0].as_ptr(), kvs[r % copies][1].as_ptr(),
-                                                   ob.as_ptr(), seq, dim, heads, heads, seq, C.c_float(dim ** -0.5))
-            for r in range(copies):
-                assert launch(r) == 0
-            stream.synchronize()
-            L.trn_event_record(e0, stream.raw())
-            for r in range(2 * copies):
-                launch(r)
-            L.trn_event_record(e1, stream.raw())
-            stream.synchronize()
-            us = elapsed_ms(e0, e1) * 1e3 / (2 * copies)
             nbytes = 8 * heads * seq * dim + 8 * heads * dim
-            attention[f"seq{seq}"] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
-                                      "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
-            for a, b in kvs:
-                a.free()
+            host = rng.standard_normal(heads * seq * dim, dtype=np.float32).view(np.uint8)
+            kb, vb = copies_of(host, nbytes // 2), copies_of(host, nbytes // 2)
+            nc = len(kb)
+            qb, ob = dp.xs[0], y[4096]
+            cold, _ = protocol(lambda r: L.trn_incremental_attention(stream.raw(), qb.as_ptr(), kb[r % nc].as_ptr(), vb[r % nc].as_ptr(),
+                                                                     ob.as_ptr(), seq, dim, heads, heads, seq, C.c_float(dim ** -0.5)),
+                               reps=100, warm=8)
+            attention[f"seq{seq}"] = {"cold": rate(nbytes, cold), "copies": nc}
+            for b in kb + vb:
                 b.free()
 
     # ---- a whole decode step: the serial layer chain with folded glue AND attention over a KV cache of 2048 -------
@@ -455,7 +424,7 @@ def main() -> int:
 
     # ---- CPU baseline: the port, layer 0's seven matrices, all host cores --------------------------
     cpu = None
-    cpu_config1 = None
+    cpu_configs = None
     if not args.no_cpu_baseline:
         from oracle.cref import CpuBaseline
         cb = CpuBaseline()
@@ -477,24 +446,29 @@ def main() -> int:
         _, sec_dq = cb.dequant_matvec("q4k", host_layer0["q"], hx[k1], k1, n1, cores, 5)
         w_f32 = kq.dequant_matrix("q4k", host_layer0["q"], n1, k1)
         _, sec_mv = cb.matvec_f32(w_f32, hx[k1], cores, 5)
-        cpu_config1 = {"shape": "Q4_K 4096x4096", "cores": cores,
-                       "dequant_matvec_us": round(sec_dq / 5 * 1e6, 1),
-                       "dequant_matvec_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_dq / 5) / 1e9, 2),
-                       "matvec_predequantised_f32_us": round(sec_mv / 5 * 1e6, 1),
-                       "matvec_predequantised_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_mv / 5) / 1e9, 2)}
+        cpu_configs = {"1_q4k_4096x4096": {"cores": cores, "dequant_matvec_us": round(sec_dq / 5 * 1e6, 1),
+                                           "dequant_matvec_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_dq / 5) / 1e9, 2),
+                                           "matvec_predequantised_f32_us": round(sec_mv / 5 * 1e6, 1),
+                                           "matvec_predequantised_gbps_quantized": round(alg_bytes("q4k", n1, k1) / (sec_mv / 5) / 1e9, 2)}}
         # configurations 2 and 3 on the CPU path (dequantise + matvec per call)
         for label, fmt, n, k in (("2_q6k_4096x4096", "q6k", 4096, 4096), ("2_q6k_32000x4096", "q6k", 32000, 4096),
                                  ("3_q5k_11008x4096", "q5k", 11008, 4096), ("3_q5k_4096x11008", "q5k", 4096, 11008)):
             wm = kq.gen_matrix(fmt, 1234 + n + k, n, k)
             _, sec = cb.dequant_matvec(fmt, wm, hx[k], k, n, cores, 3)
-            cpu_config1[label] = {"dequant_matvec_us": round(sec / 3 * 1e6, 1),
+            cpu_configs[label] = {"dequant_matvec_us": round(sec / 3 * 1e6, 1),
                                   "dequant_matvec_gbps_quantized": round(alg_bytes(fmt, n, k) / (sec / 3) / 1e9, 2)}
         cpu = {"value": round(layer_bytes * reps / spent / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"layer 0 of the pass (7 GEMVs, {layer_bytes / 1e6:.1f} MB quantized) x {reps} repetitions, "
                          f"dequantise-row + AVX2 dot, {'AVX2+FMA' if cb.has_avx2() else 'scalar'}"}
 
+    def chain(ms):
+        if ms is None:
+            return None
+        return {"us_per_pass": round(ms * 1e3, 1), "gbps": round(total_bytes / ms / 1e6, 1),
+                "frac_of_hbm_peak": round(total_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
     out = {
-        "metric": "k-quant GEMV achieved HBM GB/s (% of peak) + \u00b5s per 7B decode weight pass",
+        "metric": "k-quant GEMV achieved HBM GB/s (% of peak) + µs per 7B decode weight pass",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
@@ -502,21 +476,30 @@ def main() -> int:
                                f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} GEMVs in layer order "
                                f"(per layer x_l~N(0,1) -> q,k,v,gate,up; o<-norm(q); down<-norm(gate); head<-norm(down)), "
                                f"{total_bytes / 1e9:.3f} GB, batch 1, f32 x and y", "gemvs": len(batch),
-                               "bytes_per_step": total_bytes},
+                   "bytes_per_step": total_bytes, "launches_per_step": max(launch_of) + 1,
+                   # the same matrices in the data flow of a real decoder: every step waits for the one before it
+                   "strict_decoder_chain": chain(strict_ms) and dict(chain(strict_ms), dependent_steps=max(strict_batch.plan()) + 1),
+                   "strict_decoder_chain_with_folded_layer_glue": chain(layer_ms)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": GROUP_TRAFFIC_BYTES_PER_LAUNCH if layers == LAYERS else None,
+                     "traffic": traffic["bytes_per_launch"] if traffic else None,
+                     "traffic_measured_at": traffic.get("commit") if traffic else None,
                      "kernel": "kq_gemv_group", "launches_per_pass": n_grp,
-                     "bytes_per_launch": round(grp_bytes_per_launch), "us_per_launch": round(grp_ms * 1e3, 3)},
+                     "bytes_per_launch": round(grp_bytes_per_launch), "us_per_launch": round(grp_ms * 1e3, 3),
+                     # a launch that only reads as many bytes (trn_read_u128), same protocol: the ceiling for a launch of this size
+                     "bare_read_us_per_launch": round(read_us, 3), "bare_read_gbps": round(read_bytes / read_us / 1e3, 1),
+                     "frac_of_bare_read": round(read_us / (grp_ms * 1e3), 4)},
         "cpu_baseline": cpu,
         "extra": {"us_per_pass": round(ms_per_step * 1e3, 1), "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
                   "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
-                  "us_per_pass_strict_decoder_chain": round(strict_ms * 1e3, 1),
+                  "verification_after_timed_region_rel_l2_vs_fp64": dict(verification, tolerance=TOL),
+                  "us_per_pass_strict_decoder_chain": strict_ms and round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,
-                  "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": round(layer_ms * 1e3, 1),
-                  "per_shape_single_launch_cold": shapes, "layer_glue_us_per_launch_back_to_back": glue_us, "decode_step_7b_folded_glue_and_attention": decode_step, "f32_gemv_single_launch_cold": f32_gemv, "incremental_attention_32x128_single_launch_cold": attention,
-                  "other_configs_single_launch_cold": configs, "cpu_config1": cpu_config1,
-                  "device": ctx.device_name(), "cus": ctx.cu_count()},
+                  "weight_bytes": weight_bytes, "us_per_pass_decoder_chain_with_folded_layer_glue": layer_ms and round(layer_ms * 1e3, 1),
+                  "configs_200_launches_median_of_5": configs,
+                  "layer_glue_us_per_launch_back_to_back": glue_us, "decode_step_7b_folded_glue_and_attention": decode_step,
+                  "f32_gemv": f32_gemv, "incremental_attention_32x128": attention,
+                  "cpu_configs": cpu_configs, "device": ctx.device_name(), "cus": ctx.cu_count()},
     }
     print(json.dumps(out), flush=True)
     return 0

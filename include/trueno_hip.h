@@ -266,6 +266,10 @@ TRN_API trn_status trn_fused_residual_rmsnorm(trn_stream stream, trn_dptr residu
 /* dst[0..bytes) = src[0..bytes) with one 16-byte load and store per lane; bytes % 16 == 0.
  * The plain-copy yardstick that HBM counters are scaled by. */
 TRN_API trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t bytes);
+/* Reads src[0..bytes) once with 16-byte loads, eight in flight per lane, and stores nothing (one word of `sink`, 4 bytes,
+ * is written only if the XOR of everything read equals one particular value); bytes % 16 == 0.  The read-only
+ * yardstick: what one launch over that many bytes costs when nothing is computed.  No counterpart in the reference. */
+TRN_API trn_status trn_read_u128(trn_stream stream, trn_dptr src, uint64_t bytes, trn_dptr sink);
 TRN_API const char* trn_error_name(trn_status status);
 TRN_API const char* trn_error_string(trn_status status);
 /* Number of compute units of the current device (sizes the launches). */

@@ -71,6 +71,7 @@ SIGNATURES = {
     "trn_event_synchronize": [vp],
     "trn_event_elapsed_ms": [C.POINTER(C.c_float), vp, vp],
     "trn_copy_u128": [vp, dptr, dptr, C.c_uint64],
+    "trn_read_u128": [vp, dptr, C.c_uint64, dptr],
     "trn_error_name": [status],
     "trn_error_string": [status],
     "trn_device_cu_count": [C.POINTER(C.c_int)],

@@ -376,3 +376,25 @@ extern "C" __global__ void __launch_bounds__(256) kq_copy_u128(u32x4* dst, const
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
   for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
+
+// Read-only yardstick: every wave reads a contiguous run of 1 KB pieces, eight loads in flight per lane, nothing is
+// stored.  What a launch over so many bytes costs with no arithmetic: the ceiling the GEMV kernels are compared with.
+extern "C" __global__ void __launch_bounds__(256) kq_read_u128(const u32x4* src, uint64_t n, u32* sink) {
+  const u32 lane = threadIdx.x & 63u;
+  const uint64_t waves = (static_cast<uint64_t>(gridDim.x) * blockDim.x) >> 6;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  const uint64_t pieces = (n + 63u) / 64u, per_wave = (pieces + waves - 1u) / waves;
+  const uint64_t p0 = wave * per_wave, p1 = p0 + per_wave < pieces ? p0 + per_wave : pieces;
+  u32 acc = 0u;
+  for (uint64_t p = p0; p < p1; p += 8u) {
+    u32x4 v[8];
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      const uint64_t i = (p + d) * 64u + lane;
+      v[d] = (p + d < p1 && i < n) ? src[i] : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc ^= v[d].x ^ v[d].y ^ v[d].z ^ v[d].w;
+  }
+  if (acc == 0x9E3779B9u) *sink = acc;
+}

@@ -73,7 +73,7 @@ struct DeviceKernels {
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
-  hipFunction_t copy_u128 = nullptr;
+  hipFunction_t copy_u128 = nullptr, read_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
   hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
@@ -139,6 +139,7 @@ hipError_t device_kernels(DeviceKernels** out) {
       }
     }
     if ((e = get_fn(m, &t.copy_u128, "kq_copy_u128")) != hipSuccess ||
+        (e = get_fn(m, &t.read_u128, "kq_read_u128")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_f32_fast, "gemv_f32_fast")) != hipSuccess ||
         (e = get_fn(m, &t.q5k_from_ggml, "q5k_from_ggml")) != hipSuccess ||
         (e = get_fn(m, &t.attention, "incremental_attention")) != hipSuccess ||
@@ -1385,6 +1386,19 @@ trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t
   const uint32_t grid = uint32_t(std::min<uint64_t>((n + 255) / 256, uint64_t(d->cu_count) * 32u));
   void* args[] = {&dst, &src, &n};
   return st(hipModuleLaunchKernel(d->copy_u128, grid, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(stream), args, nullptr));
+}
+
+trn_status trn_read_u128(trn_stream stream, trn_dptr src, uint64_t bytes, trn_dptr sink) {
+  if (bytes % 16u != 0 || !aligned(src, 16) || !aligned(sink, 4)) return TRN_ERROR_INVALID_VALUE;
+  if (bytes == 0) return TRN_SUCCESS;
+  if (!src || !sink) return TRN_ERROR_INVALID_VALUE;
+  DeviceKernels* d = nullptr;
+  TRN_TRY(device_kernels(&d));
+  uint64_t n = bytes / 16u;
+  // three workgroups of four waves per CU, like the one-slab GEMV launches it is compared with
+  const uint32_t grid = uint32_t(std::min<uint64_t>((n + 255) / 256, uint64_t(d->cu_count) * 3u));
+  void* args[] = {&src, &n, &sink};
+  return st(hipModuleLaunchKernel(d->read_u128, grid, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(stream), args, nullptr));
 }
 
 const char* trn_error_name(trn_status status) {
