@@ -155,6 +155,16 @@ TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
  * one stream, or order the streams.  The kernels leave the counters at zero for the next call. */
 TRN_API trn_status trn_q4k_gemm_noalloc(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 
+/* The same products with the GEMM family's weight decode AS WRITTEN in the reference (quantize.rs:445-514 Q4_K,
+ * :727-807 Q5_K, :1009-1064 Q6_K: contiguous 12-bit scale fields normalised by 1/63, sequential nibbles, Q6_K's unsigned
+ * scales and q = ql + 4*q2 - 32), i.e. policy 1 of the dequantise surface below; the contraction is the intended one
+ * (a dot product per (row, col), quantize.rs:568-574).  trn_q*k_gemm above use the canonical (GGML) decode, so that
+ * m = 1 equals the GEMV; these exist so that q4k_gemm_ggml / q5k_gemm_ggml / q6k_gemm_ggml can be run against their
+ * as-written decode too.  Value-by-value kernels (one wave per row of W): correct, not fast. */
+TRN_API trn_status trn_q4k_gemm_as_written(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+TRN_API trn_status trn_q5k_gemm_as_written(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+TRN_API trn_status trn_q6k_gemm_as_written(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
+
 /* The legacy 18-byte-block "simplified" Q4_K GEMM, kernel name q4k_gemm_fused: W is n rows x (k/32) blocks
  * (f16 scale + 16 bytes of nibbles, w = scale * q), k a multiple of 32, C as above.  Replaces
  * QuantizeKernel::new (quantize.rs:84-93, :151-336). */

@@ -44,7 +44,7 @@ def gpu_gemv(gpu, fmt: str, buf: np.ndarray, x: np.ndarray, k: int, n: int, *, b
     return dy.copy_to_host()[:n]
 
 
-def gpu_gemm(gpu, fmt: str, buf: np.ndarray, a: np.ndarray, m: int, n: int, k: int, *, by_name=None) -> np.ndarray:
+def gpu_gemm(gpu, fmt: str, buf: np.ndarray, a: np.ndarray, m: int, n: int, k: int, *, by_name=None, as_written=False) -> np.ndarray:
     ctx, stream = gpu
     dw = t.GpuBuffer.from_host(ctx, np.ascontiguousarray(buf, np.uint8).reshape(-1))
     da = t.GpuBuffer.from_host(ctx, np.ascontiguousarray(a, np.float32).reshape(-1))
@@ -53,6 +53,6 @@ def gpu_gemm(gpu, fmt: str, buf: np.ndarray, a: np.ndarray, m: int, n: int, k: i
     if by_name is not None:
         kern.launch_by_name(stream, by_name, da, dw, dc)
     else:
-        kern.launch(stream, da, dw, dc)
+        kern.launch(stream, da, dw, dc, as_written)
     stream.synchronize()
     return dc.copy_to_host()[: m * n].reshape(m, n)

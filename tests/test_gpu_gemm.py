@@ -24,6 +24,19 @@ def test_gemm_against_fp64(gpu, fmt, n, k, m):
     assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
 
 
+@pytest.mark.parametrize("m", (1, 5))
+@pytest.mark.parametrize("fmt,n,k", [("q4k", 300, 1024), ("q5k", 300, 1024), ("q6k", 300, 2048), ("q4k", 64, 14336)])
+def test_gemm_with_the_decode_as_written(gpu, fmt, n, k, m):
+    """q*k_gemm_ggml with the GEMM family's own decode (policy 1; quantize.rs:445-514, :727-807, :1009-1064): against
+    fp64 on the oracle's as-written weights, and really different from the canonical decode's product."""
+    buf, a = kq.gen_matrix(fmt, 400 + m, n, k), kq.gen_x(500 + m, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k, as_written=True)
+    want = kq.gemm_fp64(a, kq.dequant_matrix(fmt, buf, n, k, policy=1))
+    assert c.shape == (m, n) and np.all(np.isfinite(c))
+    assert kq.rel_l2(c, want) <= TOL
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) > 1e-2
+
+
 @pytest.mark.parametrize("m", (1, 4, 16, 64))
 def test_gemm_config_shape_w_14336x4096(gpu, m):
     n, k = 14336, 4096

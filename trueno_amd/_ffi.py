@@ -50,6 +50,9 @@ SIGNATURES = {
     "trn_q4k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q5k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q6k_gemm": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
+    "trn_q4k_gemm_as_written": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
+    "trn_q5k_gemm_as_written": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
+    "trn_q6k_gemm_as_written": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q4k_gemm_noalloc": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_q4k_gemm_fused": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32, C.c_uint32],
     "trn_gemv_f32": [vp, dptr, dptr, dptr, C.c_uint32, C.c_uint32],

@@ -238,7 +238,10 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
 // ------------------------------------------------------------------------------------------
 // Batched GEMM  C[m x n] = A[m x k] . dequant(W[n x k])^T,  c[row*n + col] (quantize.rs:568-574).
 // The contraction is the intended one (a dot product per (row, col)), with the GEMV-family
-// decode, so m = 1 equals the GEMV.  VALU form: blockIdx.y walks the rows of A.
+// decode, so m = 1 equals the GEMV.  VALU form: blockIdx.y walks the rows of A.  *_gemm_as_written is the same
+// product with the GEMM family's own decode as the reference writes it (quantize.rs:445-514, :727-807, :1009-1064:
+// contiguous 12-bit scale fields normalised by 1/63, sequential nibbles, Q6_K's unsigned scales and ql + 4*q2),
+// value by value, one wave per row of W.
 // ------------------------------------------------------------------------------------------
 #define KQ_GEMM_KERNELS(fmtname, FMT)                                                                    \
   extern "C" __global__ void __launch_bounds__(512)                                                      \
@@ -257,6 +260,12 @@ extern "C" __global__ void __launch_bounds__(256) kq_fill_u32(u32* p, u32 n, u32
     for (u32 r = blockIdx.y; r < m; r += gridDim.y)                                                      \
       gemv_generic_body<FMT, POLICY_GEMV>(c + static_cast<size_t>(r) * n, b_quant,                       \
                                           a + static_cast<size_t>(r) * k, k, n, blockIdx.x, gridDim.x, 0u); \
+  }                                                                                                      \
+  extern "C" __global__ void __launch_bounds__(256)                                                      \
+      fmtname##_gemm_as_written(const float* a, const uint8_t* b_quant, float* c, u32 m, u32 n, u32 k) { \
+    for (u32 r = blockIdx.y; r < m; r += gridDim.y)                                                      \
+      gemv_generic_body<FMT, POLICY_GEMM_LEGACY>(c + static_cast<size_t>(r) * n, b_quant,                \
+                                                 a + static_cast<size_t>(r) * k, k, n, blockIdx.x, gridDim.x, 0u); \
   }
 
 KQ_GEMM_KERNELS(q4k, FMT_Q4K)

@@ -71,7 +71,7 @@ struct DeviceKernels {
   hipFunction_t fill_u32 = nullptr, gemv_group = nullptr, phases = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
-  hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {};
+  hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {}, gemm_as_written[NFMT] = {};
   hipFunction_t dequant_fast[NFMT] = {}, dequant_generic[NFMT] = {};
   hipFunction_t copy_u128 = nullptr, read_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
@@ -132,6 +132,7 @@ hipError_t device_kernels(DeviceKernels** out) {
           (e = get_fn(m, &t.gemv_generic[f], p + "_gemv_generic")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_fast[f], p + "_gemm_ggml")) != hipSuccess ||
           (e = get_fn(m, &t.gemm_generic[f], p + "_gemm_generic")) != hipSuccess ||
+          (e = get_fn(m, &t.gemm_as_written[f], p + "_gemm_as_written")) != hipSuccess ||
           (e = get_fn(m, &t.dequant_fast[f], p + "_dequant_f32")) != hipSuccess ||
           (e = get_fn(m, &t.dequant_generic[f], p + "_dequant_f32_generic")) != hipSuccess) {
         (void)hipModuleUnload(m);
@@ -432,6 +433,20 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   const uint32_t block = 256, rows_per_block = block / 64;
   const uint32_t grid = std::min<uint32_t>((n + rows_per_block - 1) / rows_per_block, uint32_t(d->cu_count) * 32u);
   return hipModuleLaunchKernel(fn, grid, is_gemv ? 1u : grid_y, 1, block, 1, 1, 0, stream, args, nullptr);
+}
+
+// The product with the GEMM family's decode as written (policy 1 of the dequantise surface): the value-by-value kernel.
+hipError_t launch_gemm_as_written(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  if (k % 256u != 0) return hipErrorInvalidValue;
+  if (n == 0 || m == 0) return hipSuccess;
+  if ((a == 0 && k != 0) || c == 0 || (w == 0 && k != 0) || !aligned(a, 4) || !aligned(c, 4)) return hipErrorInvalidValue;
+  DeviceKernels* d = nullptr;
+  hipError_t e = device_kernels(&d);
+  if (e != hipSuccess) return e;
+  const uint32_t block = 256, rows_per_block = block / 64;
+  const uint32_t grid = std::min<uint32_t>((n + rows_per_block - 1) / rows_per_block, uint32_t(d->cu_count) * 32u);
+  void* args[] = {&a, &w, &c, &m, &n, &k};
+  return hipModuleLaunchKernel(d->gemm_as_written[f], grid, std::min<uint32_t>(m, 65535u), 1, block, 1, 1, 0, stream, args, nullptr);
 }
 
 // q4k_gemm_fused: the legacy 18-byte block format (quantize.rs:151-336)
@@ -1219,6 +1234,16 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   return hipModuleLaunchKernel(d->gemv_group, first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
 }
 }  // namespace
+
+trn_status trn_q4k_gemm_as_written(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
+  return st(launch_gemm_as_written(Q4K, static_cast<hipStream_t>(s), a, b_quant, c, m, n, k));
+}
+trn_status trn_q5k_gemm_as_written(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
+  return st(launch_gemm_as_written(Q5K, static_cast<hipStream_t>(s), a, b_quant, c, m, n, k));
+}
+trn_status trn_q6k_gemm_as_written(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
+  return st(launch_gemm_as_written(Q6K, static_cast<hipStream_t>(s), a, b_quant, c, m, n, k));
+}
 
 trn_status trn_q4k_gemm_fused(trn_stream s, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k) {
   return st(launch_gemm_simplified(static_cast<hipStream_t>(s), a, b_quant, c, m, n, k));

@@ -135,8 +135,10 @@ class _GemmKernel(Kernel):
         return [C.c_uint64(_ptr(a)), C.c_uint64(_ptr(b_quant)), C.c_uint64(_ptr(c)),
                 C.c_uint32(self.m), C.c_uint32(self.n), C.c_uint32(self.k)]
 
-    def launch(self, stream: CudaStream, a, b_quant, c) -> None:
-        fn = getattr(_lib(), self._LAUNCHER)
+    def launch(self, stream: CudaStream, a, b_quant, c, as_written: bool = False) -> None:
+        """as_written: the weights decoded as the reference's GEMM kernels write it (quantize.rs:445-514, :727-807,
+        :1009-1064) instead of the canonical decode the GEMV kernels share."""
+        fn = getattr(_lib(), self._LAUNCHER + ("_as_written" if as_written else ""))
         _check(fn(stream.raw() if stream is not None else None, _ptr(a), _ptr(b_quant), _ptr(c), self.m, self.n, self.k),
                "KernelLaunch", self._NAME)
 
@@ -174,9 +176,9 @@ class QuantizeKernel(_GemmKernel):
             return super().weight_bytes()
         return self.n * self.num_blocks_per_row() * Q4K_BLOCK_BYTES
 
-    def launch(self, stream, a, b_quant, c) -> None:
+    def launch(self, stream, a, b_quant, c, as_written: bool = False) -> None:
         if self.format is Q4KFormat.GgmlSuperBlock:
-            return super().launch(stream, a, b_quant, c)
+            return super().launch(stream, a, b_quant, c, as_written)
         _check(_lib().trn_q4k_gemm_fused(stream.raw() if stream is not None else None, _ptr(a), _ptr(b_quant), _ptr(c),
                                          self.m, self.n, self.k), "KernelLaunch", self.name())
 
