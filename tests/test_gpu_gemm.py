@@ -85,68 +85,84 @@ def _tune(key, value):
     assert _ffi.lib().trn_set_tuning(key.encode(), int(value)) == 0
 
 
+MFMA_FORMATS = ("q4k", "q5k")      # the formats whose GEMM runs on the matrix cores for m >= 2
+
+
+@pytest.mark.parametrize("m", (4, 16, 64))
+@pytest.mark.parametrize("fmt", ("q5k", "q6k"))
+def test_gemm_4096x4096(gpu, fmt, m):
+    n = k = 4096
+    buf, a = kq.gen_matrix(fmt, 1239, n, k), kq.gen_x(4321, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
+
+
 @pytest.mark.parametrize("m", (2, 9, 13, 33))
 @pytest.mark.parametrize("n,k", [(100, 512), (1000, 2304)])
-def test_q4k_gemm_matrix_core_form_ragged(gpu, n, k, m):
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_matrix_core_form_ragged(gpu, fmt, n, k, m):
     """Token counts that do not fill a tile of 16, row counts that do not fill a strip of 32 or a group of 8 strips."""
-    buf, a = kq.gen_matrix("q4k", 50 + m, n, k), kq.gen_x(60 + m, m, k)
-    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
-    assert kq.rel_l2(c, _c64("q4k", buf, a, n, k)) <= TOL
+    buf, a = kq.gen_matrix(fmt, 50 + m, n, k), kq.gen_x(60 + m, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
 
 
-def test_q4k_gemm_parts_of_k(gpu):
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_parts_of_k(gpu, fmt):
     """However K is cut into parts the result stays within tolerance, and the same cut gives the same bits on
     every run: the parts are added in part order by whichever workgroup arrives last."""
     n, k, m = 777, 2048, 24
-    buf, a = kq.gen_matrix("q4k", 91, n, k), kq.gen_x(92, m, k)
-    c64 = _c64("q4k", buf, a, n, k)
+    buf, a = kq.gen_matrix(fmt, 91, n, k), kq.gen_x(92, m, k)
+    c64 = _c64(fmt, buf, a, n, k)
     try:
         for waves in (4, 8):
             _tune("gemm_waves", waves)
             for parts in (1, 2, 3, 8):
                 _tune("gemm_k_parts", parts)
-                first = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+                first = gpu_gemm(gpu, fmt, buf, a, m, n, k)
                 assert kq.rel_l2(first, c64) <= TOL
                 for _ in range(3):
-                    again = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+                    again = gpu_gemm(gpu, fmt, buf, a, m, n, k)
                     assert np.array_equal(again.view(np.uint32), first.view(np.uint32)), (waves, parts)
     finally:
         _tune("gemm_k_parts", 0)
         _tune("gemm_waves", 0)
     try:
         _tune("gemm_mfma_off", 1)
-        valu = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+        valu = gpu_gemm(gpu, fmt, buf, a, m, n, k)
     finally:
         _tune("gemm_mfma_off", 0)
     assert kq.rel_l2(valu, c64) <= TOL
 
 
-def test_q4k_gemm_no_worse_than_reference_order_f32(gpu):
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_no_worse_than_reference_order_f32(gpu, fmt):
     """Per token, the error against fp64 stays within the slack of an f32 evaluation in the reference's
     summation order (quantize.rs:1412-1518)."""
     n, k, m = 512, 4096, 16
-    buf, a = kq.gen_matrix("q4k", 93, n, k), kq.gen_x(94, m, k)
-    w = kq.dequant_matrix("q4k", buf, n, k)
-    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    buf, a = kq.gen_matrix(fmt, 93, n, k), kq.gen_x(94, m, k)
+    w = kq.dequant_matrix(fmt, buf, n, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
     c64 = kq.gemm_fp64(a, w)
     ref = np.stack([kq.gemv_ref_order_fp32(w, a[i]) for i in range(m)])
     err_ref, err_ours = kq.rel_l2(ref, c64), kq.rel_l2(c, c64)
-    print(f"q4k gemm {m}x{n}x{k}: ours {err_ours:.3e} vs reference-order f32 {err_ref:.3e}")
+    print(f"{fmt} gemm {m}x{n}x{k}: ours {err_ours:.3e} vs reference-order f32 {err_ref:.3e}")
     assert err_ours <= 1.5 * err_ref + 1e-9
 
 
-def test_q4k_gemm_special_values(gpu):
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_special_values(gpu, fmt):
     """An all-zero token, a huge and a tiny token, and a token with an infinity (its outputs are not finite,
     the other tokens are untouched)."""
     n, k, m = 64, 512, 5
-    buf = kq.gen_matrix("q4k", 95, n, k)
+    buf = kq.gen_matrix(fmt, 95, n, k)
     a = kq.gen_x(96, m, k)
     a[1] = 0.0
     a[2] *= 1e30
     a[3] *= 1e-30
     a[4, 17] = np.inf
-    c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
-    w = kq.dequant_matrix("q4k", buf, n, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    w = kq.dequant_matrix(fmt, buf, n, k)
     c64 = kq.gemm_fp64(a[:4], w)
     assert np.all(c[1] == 0.0)
     for i in (0, 2, 3):

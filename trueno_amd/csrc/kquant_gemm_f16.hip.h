@@ -1,7 +1,13 @@
-// Batched Q4_K GEMM on the matrix cores (gfx950, v_mfma_f32_32x32x16_f16).
+// Batched Q4_K / Q5_K GEMM on the matrix cores (gfx950, v_mfma_f32_32x32x16_f16).
 //
 //   C[m x n] = A[m x k] . dequant(W[n x k])^T,  c[row*n + col]      (trueno-gpu/src/kernels/quantize.rs:568-574,
-//   decode of the weights as in the GEMV family, quantize.rs:1237-1483)
+//   decode of the weights as in the GEMV family, quantize.rs:1237-1483 Q4_K, :1589-1693 Q5_K)
+//
+// Q5_K (the reference's layout: nibbles as Q4_K, eight contiguous 12-bit (scale, min) fields, fifth bit of value i in
+// bit i%8 of qh[i/8] at byte 144) runs through the same kernel: q <= 31 and s_j <= 63 keep q * s_j below 2048, still
+// exact in f16; the fifth bits are joined into the nibbles' 16-bit lanes before the packed multiply (a 5-bit quant in
+// the low bits of a 16-bit lane is still the subnormal q * 2^-24); rows of 176 bytes are 11 sixteen-byte pieces, an odd
+// stride like Q4_K's 9, so the transposed reads stay conflict-free.
 //
 // f16 operands without giving up f32 accuracy:
 //   * the weight operand is  q * s_j * 2^-14  (nibble q <= 15, 6-bit sub-block scale s_j <= 63): an integer
@@ -49,9 +55,13 @@ constexpr u32 kXpMainBytes = 16 * 1024;        // 16 products x 64 lanes x 16 by
 constexpr u32 kXpSumBytes = 512;               // 64 lanes x 4 f16
 constexpr u32 kXpFactorBytes = 64;             // 16 tokens x f32
 constexpr u32 kXpStageBytes = kXpMainBytes + kXpSumBytes + kXpFactorBytes;
-constexpr u32 kWStageBytes = 32 * 144;         // one super-block of 32 rows
+// weight tile of one super-block of 32 rows: SB bytes a row, PIECES sixteen-byte pieces a row, copied by DMA instructions
+// of 64 pieces each (the last one half full for both formats: 288 = 4.5 x 64, 352 = 5.5 x 64)
+template <int FMT> struct WTile;
+template <> struct WTile<FMT_Q4K> { static constexpr u32 SB = 144, PIECES = 9, DMA = 5, BYTES = 32 * 144; };
+template <> struct WTile<FMT_Q5K> { static constexpr u32 SB = 176, PIECES = 11, DMA = 6, BYTES = 32 * 176; };
 // dynamic LDS: two stages of token operands, two weight tiles per wave, one word for the arrival order
-__host__ __device__ constexpr u32 lds_bytes(u32 waves) { return 2u * kXpStageBytes + 2u * waves * kWStageBytes + 16u; }
+__host__ __device__ constexpr u32 lds_bytes(u32 waves, u32 tile_bytes) { return 2u * kXpStageBytes + 2u * waves * tile_bytes + 16u; }
 
 __device__ __forceinline__ u32 wave_max_u32(u32 v) {
   v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true)));
@@ -165,8 +175,8 @@ __device__ __forceinline__ h16x2 pk_mul_h2(u32 bits, h16x2 s) { return as_h16x2(
 // at the (group, tile) counter adds the parts in part order - the sum does not depend on who is last - and
 // puts the counter back to zero (the counters start at zero when the workspace is allocated).
 //   dynamic LDS = kLdsBytes
-template <int CHUNKS>     // chunks of A a thread converts per super-block: 512 / threads
-__device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
+template <int FMT, int CHUNKS>     // CHUNKS: chunks of A a thread converts per super-block, 512 / threads
+__device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
                                          u32* __restrict__ counters, u32 m, u32 n, u32 nsb, u32 ksb, u32 kparts,
                                          u32 groups, u32 tiles, u32 lds_base) {
   const u32 lane = threadIdx.x & 63u;
@@ -179,14 +189,17 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
   const u32 waves = blockDim.x >> 6;
   const u32 strip = group * waves + wave;
   const u32 col = lane & 31u, g = lane >> 5;
-  const size_t row_bytes = static_cast<size_t>(nsb) * 144u;
+  using T = WTile<FMT>;
+  constexpr u32 kWStageBytes = T::BYTES;
+  constexpr int DMA = static_cast<int>(T::DMA);
+  const size_t row_bytes = static_cast<size_t>(nsb) * T::SB;
 
-  // where this lane's pieces of a weight tile come from: piece p = 64 t + lane of [32 rows][9 pieces]
-  size_t woff[5];
+  // where this lane's pieces of a weight tile come from: piece p = 64 t + lane of [32 rows][PIECES pieces]
+  size_t woff[DMA];
 #pragma unroll
-  for (int t = 0; t < 5; ++t) {
-    const u32 p = min(64u * t + lane, 287u);
-    const u32 r = p / 9u, cc = p - 9u * r;
+  for (int t = 0; t < DMA; ++t) {
+    const u32 p = min(64u * t + lane, 32u * T::PIECES - 1u);
+    const u32 r = p / T::PIECES, cc = p - T::PIECES * r;
     woff[t] = static_cast<size_t>(min(strip * 32u + r, n - 1u)) * row_bytes + 16u * cc;
   }
   const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * (2u * kWStageBytes);
@@ -206,15 +219,13 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
     live[i] = token < m;
   }
 
-  // Loads are counted by hand (s_waitcnt vmcnt): per super-block a wave issues 2*CHUNKS loads of A, then 5 of W.
+  // Loads are counted by hand (s_waitcnt vmcnt): per super-block a wave issues 2*CHUNKS loads of A, then DMA of W.
   auto issue_w = [&](u32 s) {
-    const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * 144u;
+    const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * T::SB;
     const u32 wl = lds_w + (s & 1u) * kWStageBytes;
-    dma16(wsrc + woff[0], wl);
-    dma16(wsrc + woff[1], wl + 1024u);
-    dma16(wsrc + woff[2], wl + 2048u);
-    dma16(wsrc + woff[3], wl + 3072u);
-    if (lane < 32u) dma16(wsrc + woff[4], wl + 4096u);
+#pragma unroll
+    for (int t = 0; t < DMA - 1; ++t) dma16(wsrc + woff[t], wl + 1024u * t);
+    if (lane < 32u) dma16(wsrc + woff[DMA - 1], wl + 1024u * (DMA - 1));
   };
   u32x4 an[CHUNKS][2];                 // A of a super-block on its way to conversion
   auto load_a = [&](u32 s) {
@@ -225,9 +236,9 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
                    : "=&v"(an[i][0]), "=&v"(an[i][1]) : "v"(src) : "memory");
     }
   };
-  auto convert = [&](u32 s) {          // the loads of A issued last have landed when 5 loads (of W) are left
+  auto convert = [&](u32 s) {          // the loads of A issued last have landed when DMA loads (of W) are left
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) asm volatile("s_waitcnt vmcnt(5)" : "+v"(an[i][0]), "+v"(an[i][1])::"memory");
+    for (int i = 0; i < CHUNKS; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA) : "memory");
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i)
@@ -251,11 +262,11 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
   }
   for (u32 s = 0; s < ns; ++s) {
     // weight tile s has landed (the loads of super-block s+1 may be in flight); the token operands of s are written
-    if (s + 1u < ns) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * CHUNKS + 5) : "memory");
+    if (s + 1u < ns) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * CHUNKS + DMA) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
     const u32 slot = s & 1u;
-    const u32 wt = lds_w + slot * kWStageBytes + col * 144u, wl = wt + g * 64u;
+    const u32 wt = lds_w + slot * kWStageBytes + col * T::SB, wl = wt + g * 64u;
     const u32 xl = lds_xp + slot * kXpStageBytes + lane * 16u;
     const u32 sl = lds_xp + slot * kXpStageBytes + kXpMainBytes + lane * 8u;
     const u32 fl = lds_xp + slot * kXpStageBytes + kXpMainBytes + kXpSumBytes + g * 8u;
@@ -271,8 +282,10 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
     lds_read64<16>(f23, fl);
     lds_read64<32>(f45, fl);
     lds_read64<48>(f67, fl);
+    [[maybe_unused]] u32x4 qh = {0u, 0u, 0u, 0u};      // Q5_K: this lane group's 16 bytes of fifth bits (values 128 g .. 128 g + 127)
+    if constexpr (FMT == FMT_Q5K) lds_read128<144>(qh, wt + g * 16u);
     lds_wait5(hdr, d0, d1, d2, d3, sx);
-    asm volatile("" : "+v"(f01), "+v"(f23), "+v"(f45), "+v"(f67));
+    asm volatile("" : "+v"(f01), "+v"(f23), "+v"(f45), "+v"(f67), "+v"(qh));
     if (s + 1u < ns) convert(s + 1u);        // into the stage that was read two super-blocks ago
     if (s + 2u < ns) {          // the weight tile is in registers: its LDS space takes the tile after the next
       load_a(s + 2u);
@@ -280,9 +293,18 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
     }
     const u32 dw[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w, d2.x, d2.y, d2.z, d2.w, d3.x, d3.y, d3.z, d3.w};
     const float d = half_bits_to_f32(hdr.x), dmin = half_bits_to_f32(hdr.x >> 16);
-    // this lane's four 6-bit scales and mins as bytes (get_scale_min_k4, quantize.rs:1306-1385)
-    const u32 s4 = g ? ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u)) : (hdr.y & 0x3F3F3F3Fu);
-    const u32 m4 = g ? (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u)) : (hdr.z & 0x3F3F3F3Fu);
+    // this lane's four 6-bit scales and mins (sub-blocks 4g .. 4g+3) as bytes
+    u32 s4, m4;
+    if constexpr (FMT == FMT_Q4K) {      // get_scale_min_k4, quantize.rs:1306-1385
+      s4 = g ? ((hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u)) : (hdr.y & 0x3F3F3F3Fu);
+      m4 = g ? (((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u)) : (hdr.z & 0x3F3F3F3Fu);
+    } else {                             // eight contiguous 12-bit fields, scale in the low six bits (quantize.rs:1607-1635)
+      const u32 lo = g ? ((hdr.z >> 16) | (hdr.w << 16)) : hdr.y;      // fields 4g, 4g+1 and the low byte of 4g+2
+      const u32 hi = g ? (hdr.w >> 16) : (hdr.z & 0xFFFFu);            // the rest of field 4g+2 and field 4g+3
+      const u32 f0 = lo & 0xFFFu, f1 = (lo >> 12) & 0xFFFu, f2 = ((lo >> 24) | (hi << 8)) & 0xFFFu, f3 = (hi >> 4) & 0xFFFu;
+      s4 = (f0 & 63u) | ((f1 & 63u) << 8) | ((f2 & 63u) << 16) | ((f3 & 63u) << 24);
+      m4 = (f0 >> 6) | ((f1 >> 6) << 8) | ((f2 >> 6) << 16) | ((f3 >> 6) << 24);
+    }
     h16x2 sc[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -314,14 +336,30 @@ __device__ __forceinline__ void q4k_body(const float* __restrict__ a, const uint
         const int u = uu + i;
         const u32 t0 = dw[2 * u], t1 = dw[2 * u + 1], t0s = t0 >> 8, t1s = t1 >> 8;
         const h16x2 sl2 = sc[(u >> 2) * 2], sh2 = sc[(u >> 2) * 2 + 1];
-        bl[i][0] = __builtin_bit_cast(u32, pk_mul_h2(t0 & 0x000F000Fu, sl2));
-        bl[i][1] = __builtin_bit_cast(u32, pk_mul_h2(t0s & 0x000F000Fu, sl2));
-        bl[i][2] = __builtin_bit_cast(u32, pk_mul_h2(t1 & 0x000F000Fu, sl2));
-        bl[i][3] = __builtin_bit_cast(u32, pk_mul_h2(t1s & 0x000F000Fu, sl2));
-        bh[i][0] = __builtin_bit_cast(u32, pk_mul_h2(t0 & 0x00F000F0u, sh2));
-        bh[i][1] = __builtin_bit_cast(u32, pk_mul_h2(t0s & 0x00F000F0u, sh2));
-        bh[i][2] = __builtin_bit_cast(u32, pk_mul_h2(t1 & 0x00F000F0u, sh2));
-        bh[i][3] = __builtin_bit_cast(u32, pk_mul_h2(t1s & 0x00F000F0u, sh2));
+        // Q5_K: the fifth bits of the eight values of dword j (j = 2u, 2u+1) are nibble j%8 of qh word 2(j/8) (low
+        // nibbles) and 2(j/8)+1 (high nibbles), bit i for byte i.  n * (2^4 + 2^18) puts bit 0 at bit 4 and bit 2 at
+        // bit 20 - where the fifth bit of a low nibble's 16-bit lane belongs for bytes 0 and 2 -, n * (2^3 + 2^17) the
+        // same for bytes 1 and 3; for the high nibbles (quant in bits 4..7 of its lane) four places further up.
+        u32 f[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}}, e[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        if constexpr (FMT == FMT_Q5K) {
+          const u32 ql5 = u < 4 ? qh.x : qh.z, qh5 = u < 4 ? qh.y : qh.w;
+#pragma unroll
+          for (int d = 0; d < 2; ++d) {
+            const u32 nl = (ql5 >> (4 * ((2 * u + d) & 7))) & 15u, nh = (qh5 >> (4 * ((2 * u + d) & 7))) & 15u;
+            f[d][0] = __umul24(nl, 0x40010u) & 0x00100010u;      // low nibbles, bytes 0 and 2
+            f[d][1] = __umul24(nl, 0x20008u) & 0x00100010u;      // low nibbles, bytes 1 and 3
+            e[d][0] = __umul24(nh, 0x400100u) & 0x01000100u;     // high nibbles, bytes 0 and 2
+            e[d][1] = __umul24(nh, 0x200080u) & 0x01000100u;     // high nibbles, bytes 1 and 3
+          }
+        }
+        bl[i][0] = __builtin_bit_cast(u32, pk_mul_h2((t0 & 0x000F000Fu) | f[0][0], sl2));
+        bl[i][1] = __builtin_bit_cast(u32, pk_mul_h2((t0s & 0x000F000Fu) | f[0][1], sl2));
+        bl[i][2] = __builtin_bit_cast(u32, pk_mul_h2((t1 & 0x000F000Fu) | f[1][0], sl2));
+        bl[i][3] = __builtin_bit_cast(u32, pk_mul_h2((t1s & 0x000F000Fu) | f[1][1], sl2));
+        bh[i][0] = __builtin_bit_cast(u32, pk_mul_h2((t0 & 0x00F000F0u) | e[0][0], sh2));
+        bh[i][1] = __builtin_bit_cast(u32, pk_mul_h2((t0s & 0x00F000F0u) | e[0][1], sh2));
+        bh[i][2] = __builtin_bit_cast(u32, pk_mul_h2((t1 & 0x00F000F0u) | e[1][0], sh2));
+        bh[i][3] = __builtin_bit_cast(u32, pk_mul_h2((t1s & 0x00F000F0u) | e[1][1], sh2));
       }
       lds_wait4(a0, a1, a2, a3);
 #pragma unroll

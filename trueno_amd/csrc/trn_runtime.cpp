@@ -76,7 +76,7 @@ struct DeviceKernels {
   hipFunction_t copy_u128 = nullptr, read_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
-  hipFunction_t gemm_f16[2] = {};   // 4 and 8 strips per workgroup
+  hipFunction_t gemm_f16[2][2] = {};   // [Q4_K, Q5_K][4 or 8 strips per workgroup]
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
@@ -153,8 +153,10 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
         (e = get_fn(m, &t.dequant_simplified, "q4k_simplified_dequant_f32")) != hipSuccess ||
-        (e = get_fn(m, &t.gemm_f16[0], "q4k_gemm_f16_w4")) != hipSuccess ||
-        (e = get_fn(m, &t.gemm_f16[1], "q4k_gemm_f16_w8")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[0][0], "q4k_gemm_f16_w4")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[0][1], "q4k_gemm_f16_w8")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[1][0], "q5k_gemm_f16_w4")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[1][1], "q5k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -362,14 +364,15 @@ hipError_t launch_attention(hipStream_t stream, uint64_t q, uint64_t k, uint64_t
 // demand and kept.  The counters are zero between products: the kernel puts them back.
 ScratchMap g_gemm_ws;
 
-constexpr uint32_t kGemmXpStageBytes = 16 * 1024 + 512 + 64, kGemmWTileBytes = 32 * 144;
+constexpr uint32_t kGemmXpStageBytes = 16 * 1024 + 512 + 64;
 constexpr size_t kGemmCounterBytes = size_t(1) << 16;   // arrival counters at the front of the GEMM's scratch buffer
 
 // ext_base != 0: the caller brings the scratch buffer (ext_cap bytes, counters at its front already zero); nothing is
 // allocated and a product that needs more is refused.
-hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
-                               uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0) {
+hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
+                              uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
+  const uint32_t kGemmWTileBytes = 32u * kSbBytes[f];
   // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
   const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
   const uint32_t lds = 2u * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
@@ -399,13 +402,24 @@ hipError_t launch_q4k_gemm_f16(DeviceKernels* d, hipStream_t stream, uint64_t a,
   const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
   uint32_t nsb_arg = nsb, ksb_arg = ksb, kparts_arg = kparts, groups_arg = groups, tiles_arg = tiles;
   void* margs[] = {&a, &w, &c, &part, &cnt, &m, &n, &nsb_arg, &ksb_arg, &kparts_arg, &groups_arg, &tiles_arg};
-  return hipModuleLaunchKernel(d->gemm_f16[waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
+  return hipModuleLaunchKernel(d->gemm_f16[f == Q5K][waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
-// does the matrix-core form take this product?
+// does the matrix-core form take this product?  (Q4_K and Q5_K)
 bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
   return m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
          uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u;   // its arrival counters
+}
+
+// A few tokens against a small matrix are faster through the GEMV engine, one pass per token with the weights of the
+// second and later passes coming from the caches, than through the matrix-core kernel with its start-up and its sum
+// over the parts of K.  Times in microseconds fitted to measurements on MI355X (MB = weight bytes / 1e6):
+//   engine: 3.9 + MB / 5.7 for the first token, MB / 7 + 0.4 for each further one (one slab of columns only; with
+//   k > 4096 a further pass costs as much as the first); matrix cores: 12 + MB / 9.4 for up to 16 tokens.
+bool gemm_few_tokens_by_engine(Fmt f, uint32_t m, uint32_t n, uint32_t k) {
+  if (m > 8u || k > 4096u) return false;
+  const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
+  return 3.9 + mb / 5.7 + (m - 1u) * (mb / 7.0 + 0.4) < 12.0 + mb / 9.4;
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
@@ -416,7 +430,9 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
-  if (!is_gemv && f == Q4K && q4k_gemm_f16_ok(a, w, c, m, n, k)) return launch_q4k_gemm_f16(d, stream, a, w, c, m, n, k);
+  if (!is_gemv && (f == Q4K || f == Q5K) && q4k_gemm_f16_ok(a, w, c, m, n, k) &&
+      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || !gemm_few_tokens_by_engine(f, m, n, k)))
+    return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
@@ -1343,7 +1359,9 @@ trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c
   if (n == 0 || m == 0) return TRN_SUCCESS;
   if ((a == 0 && k != 0) || c == 0 || (b == 0 && k != 0)) return TRN_ERROR_INVALID_VALUE;
   hipStream_t stream = static_cast<hipStream_t>(s);
-  if (!q4k_gemm_f16_ok(a, b, c, m, n, k)) return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));  // no scratch at all
+  // the same choice of kernel as trn_q4k_gemm, so the same bits: the GEMV engine needs no scratch at all
+  if (!q4k_gemm_f16_ok(a, b, c, m, n, k) || (g_tune_gemm_ksplit == 0 && g_tune_gemm_waves == 0 && gemm_few_tokens_by_engine(Q4K, m, n, k)))
+    return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));
   DeviceKernels* d = nullptr;
   TRN_TRY(device_kernels(&d));
   int dev = 0;
@@ -1352,7 +1370,7 @@ trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c
   const uint64_t base = trn_noalloc_scratch(dev, &cap);
   if (!base) return TRN_ERROR_INVALID_VALUE;
   // launch_q4k_gemm_f16 answers hipErrorInvalidValue when the product needs more than `cap`: name that case
-  const hipError_t e = launch_q4k_gemm_f16(d, stream, a, b, c, m, n, k, base, cap);
+  const hipError_t e = launch_kq_gemm_f16(d, Q4K, stream, a, b, c, m, n, k, base, cap);
   if (e == hipErrorInvalidValue) return TRN_ERROR_SCRATCH_TOO_SMALL;
   return st(e);
 }
