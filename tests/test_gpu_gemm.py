@@ -85,7 +85,7 @@ def _tune(key, value):
     assert _ffi.lib().trn_set_tuning(key.encode(), int(value)) == 0
 
 
-MFMA_FORMATS = ("q4k", "q5k")      # the formats whose GEMM runs on the matrix cores for m >= 2
+MFMA_FORMATS = ("q4k", "q5k", "q6k")      # the formats whose GEMM runs on the matrix cores for m >= 2
 
 
 @pytest.mark.parametrize("m", (4, 16, 64))

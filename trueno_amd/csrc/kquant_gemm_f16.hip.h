@@ -42,6 +42,7 @@
 // the loads in flight.
 #pragma once
 #include "kquant_common.hip.h"
+#include <type_traits>
 
 typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
@@ -111,8 +112,9 @@ __device__ __forceinline__ void dma16(const uint8_t* src, u32 lds_addr) {
 __device__ __forceinline__ void lds_write128x2(u32 addr, const u32x4& a, const u32x4& b) {
   asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:16" ::"v"(addr), "v"(a), "v"(b) : "memory");
 }
-__device__ __forceinline__ void lds_write16x2(u32 addr, u32 a, u32 b) {     // the low halves of a and b, 8 bytes apart
-  asm volatile("ds_write_b16 %0, %1\n\tds_write_b16 %0, %2 offset:8" ::"v"(addr), "v"(a), "v"(b) : "memory");
+template <int APART>
+__device__ __forceinline__ void lds_write16x2(u32 addr, u32 a, u32 b) {     // the low halves of a and b, APART bytes apart
+  asm volatile("ds_write_b16 %0, %1\n\tds_write_b16 %0, %2 offset:%3" ::"v"(addr), "v"(a), "v"(b), "n"(APART) : "memory");
 }
 __device__ __forceinline__ void lds_write32(u32 addr, u32 a) { asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(a) : "memory"); }
 
@@ -124,6 +126,8 @@ __device__ __forceinline__ void lds_write32(u32 addr, u32 a) { asm volatile("ds_
 //                                               holds an infinity or a NaN)
 // This thread brings the eight elements 8c .. 8c+7 (v0, v1) of token `token` of the tile; the 32 threads of a
 // half wave hold one token's run.
+// SUMS = false (Q6_K, whose kernel needs no sums) leaves the sums out.
+template <bool SUMS = true>
 __device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, u32 token, u32 c, u32 stage) {
   const u32 lane = threadIdx.x & 63u;
   const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
@@ -156,18 +160,94 @@ __device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, 
   // the 16 products' pages are 1 KB apart, i.e. on the same banks: slot s of page q lies at s ^ 2q, so that the lanes
   // of a token, which write the same slot of different pages, do not all hit one bank (the reader applies the same)
   lds_write128x2(stage + q * 1024u + ((32u * g + 2u * token) ^ (2u * q)) * 16u, ph, pl);
-  float sj = ((xs[0] + xs[1]) + (xs[2] + xs[3])) + ((xs[4] + xs[5]) + (xs[6] + xs[7]));
-  sj += dpp_f32<0xB1>(sj);
-  sj += dpp_f32<0x4E>(sj);                  // the four threads of a sub-block hold its sum
-  if ((c & 3u) == 0u) {
-    _Float16 sh, sl;
-    split_f16(sj * 0.03125f, sh, sl);
-    lds_write16x2(stage + kXpMainBytes + (32u * g + 2u * token) * 8u + 2u * (j & 3u), pack_h2(sh, sh), pack_h2(sl, sl));
+  if constexpr (SUMS) {
+    float sj = ((xs[0] + xs[1]) + (xs[2] + xs[3])) + ((xs[4] + xs[5]) + (xs[6] + xs[7]));
+    sj += dpp_f32<0xB1>(sj);
+    sj += dpp_f32<0x4E>(sj);                // the four threads of a sub-block hold its sum
+    if ((c & 3u) == 0u) {
+      _Float16 sh, sl;
+      split_f16(sj * 0.03125f, sh, sl);
+      lds_write16x2<8>(stage + kXpMainBytes + (32u * g + 2u * token) * 8u + 2u * (j & 3u), pack_h2(sh, sh), pack_h2(sl, sl));
+    }
   }
   if (c == 0u) lds_write32(stage + kXpMainBytes + kXpSumBytes + 4u * token, finite ? (eb << 23) : 0x7FC00000u);
 }
 
 __device__ __forceinline__ h16x2 pk_mul_h2(u32 bits, h16x2 s) { return as_h16x2(bits) * s; }
+__device__ __forceinline__ h16x2 pk_fma_h2(u32 bits, h16x2 s, h16x2 add) { return __builtin_elementwise_fma(as_h16x2(bits), s, add); }
+
+// What the kernels do with a finished tile.  lane l, tot registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row
+// strip*32 + col.  With one part of K the result is stored; otherwise the part is published and the workgroup that
+// arrives last at the (group, tile) counter adds the parts in part order and puts the counter back to zero.
+__device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict__ c, float* __restrict__ partial, u32* __restrict__ counters,
+                                            u32 m, u32 n, u32 kparts, u32 groups, u32 tiles, u32 waves, u32 group, u32 part, u32 tile,
+                                            u32 strip, u32 col, u32 g, u32 lane, u32 lds_flag) {
+  // lane l, registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row strip*32 + col
+  const u32 row = strip * 32u + col;
+  const bool row_ok = row < n;
+  const u32 tokens_pad = tiles * kTokensPerTile;
+  float val[8];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) val[2 * a + b] = fmaf(tot[4 * a + 2 * b + 1], 0.00048828125f, tot[4 * a + 2 * b]);
+  if (kparts == 1u) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
+        if (row_ok && token < m) c[static_cast<size_t>(token) * n + row] = val[2 * a + b];
+      }
+    return;
+  }
+  // several parts of K: publish this part, the last arrival adds them up.  The parts cross workgroups (and XCDs):
+  // 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side by side:
+  //   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
+  const u32 strips = groups * waves;
+  const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      partial, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
+  auto slot_of = [&](u32 pt) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
+  __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[0]), __float_as_uint(val[1]), __float_as_uint(val[2]), __float_as_uint(val[3])},
+                                         part_rsrc, slot_of(part), 0, 16);
+  const bool upper = tile * kTokensPerTile + 8u < m;      // tokens 8..15 of the tile exist (val[4..7])
+  if (upper)
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[4]), __float_as_uint(val[5]), __float_as_uint(val[6]), __float_as_uint(val[7])},
+                                           part_rsrc, slot_of(part) + 16, 0, 16);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
+  asm volatile("s_barrier" ::: "memory");
+  if (threadIdx.x == 0u) {
+    const u32 old = __hip_atomic_fetch_add(counters + group * tiles + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(lds_flag), "v"(old) : "memory");
+  }
+  asm volatile("s_barrier" ::: "memory");
+  u32 old;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(lds_flag) : "memory");
+  if (old == kparts - 1u && threadIdx.x == 0u)      // ready for the next product on this stream
+    __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (old != kparts - 1u || !row_ok) return;
+  float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // eight parts in flight, added in part order
+    u32x4 lo[8], hi[8];
+#pragma unroll
+    for (u32 pp = 0; pp < 8; ++pp) {
+      const u32 pt = min(p0 + pp, kparts - 1u);
+      lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
+      hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (u32 pp = 0; pp < 8; ++pp)
+      if (p0 + pp < kparts) {
+        r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
+        r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
+      }
+  }
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
+    if (token < m) c[static_cast<size_t>(token) * n + row] = r[t];
+  }
+}
 
 // Main kernel.  Workgroup id -> (unit, token tile) with the token tiles of a unit 8 ids apart (same XCD, so the
 // weights they share meet in that XCD's L2); unit -> (group of 8 strips, part of K).  With one part the result
@@ -380,71 +460,239 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     }
   }
 
-  // lane l, registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row strip*32 + col
-  const u32 row = strip * 32u + col;
-  const bool row_ok = row < n;
-  const u32 tokens_pad = tiles * kTokensPerTile;
-  float val[8];
+  finish_tile(tot, c, partial, counters, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
+}
+
+
+// ------------------------------------------------------------------------------------------------------------
+// Q6_K (quantize.rs:1806-1934: ql[128] @0, qh[64] @128, sc[16] int8 @192, d f16 @208; w = d * sc * (q - 32) with
+// q = nibble | (two bits of qh) << 4, scales per 16 values) on the matrix cores.
+//   * (q - 32) * sc needs 13 bits: not exact in f16.  With centred digits  q - 32 = (nib - 8) + 8 (2 q2 - 3)  the two
+//     products (nib - 8) sc (at most 8 * 128) and (2 q2 - 3) sc (at most 3 * 128) are exact operands, neither is large
+//     against the value they add up to, and no sum of the tokens is needed.  Both come from the bits in place as for
+//     Q4_K: a nibble or a 2-bit field moved to bits 4..7 of its 16-bit lane is the subnormal v * 2^-20; one packed
+//     multiply-add with (sc * 2^6, -8 sc * 2^-14), or (sc * 2^7, -3 sc * 2^-14), gives the operand times 2^-14.  Two
+//     accumulators over the super-block are combined per (row, token, super-block):  tot += d * 2^E * (acc_n + 8 acc_q).
+//   * lane group g = l/32 of W row r takes half g of the super-block (values 128g .. 128g+127: ql[64g ..], qh[32g ..],
+//     sc[8g ..]).  Token page Q of the Q4_K layout (values 128g + 64(U/4) + 32(Q%2) + 8(U%4) + .., U = Q/2) holds the
+//     eight values that the low (U/4 = 0) or high nibbles of ql dwords 8(Q%2) + 2(U%4) + {0, 1} and field 2(U/4) + Q%2 of
+//     qh dwords 2(U%4) + {0, 1} belong to: one read of a token page feeds two products.
+//   * blocks of 210 bytes are only 2-byte aligned, which the copy into LDS by DMA does not take: the weight tile of
+//     the NEXT super-block travels through registers (13 sixteen-byte loads and one 2-byte load per row, issued a
+//     super-block ahead, written to LDS when the current one's products are done; rows 240 bytes apart in LDS, 15 pieces).
+// Everything else (token conversion, parts of K, the sum over the parts) is the Q4_K kernel's.
+constexpr u32 kQ6RowStride = 240u;                         // LDS bytes between the rows of a weight tile
+constexpr u32 kQ6TileBytes = 32u * kQ6RowStride;
+__host__ __device__ constexpr u32 q6k_lds_bytes(u32 waves) { return 2u * kXpStageBytes + waves * kQ6TileBytes + 16u; }
+
+template <int CHUNKS>
+__device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
+                                         u32* __restrict__ counters, u32 m, u32 n, u32 nsb, u32 ksb, u32 kparts,
+                                         u32 groups, u32 tiles, u32 lds_base) {
+  const u32 lane = threadIdx.x & 63u;
+  const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
+  const u32 id = blockIdx.x;
+  const u32 unit = (id / (8u * tiles)) * 8u + (id & 7u), tile = (id >> 3) % tiles;
+  if (unit >= groups * kparts) return;
+  const u32 group = unit / kparts, part = unit - group * kparts;
+  const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
+  const u32 waves = blockDim.x >> 6;
+  const u32 strip = group * waves + wave;
+  const u32 col = lane & 31u, g = lane >> 5;
+  const size_t row_bytes = static_cast<size_t>(nsb) * 210u;
+
+  // this lane's pieces of a weight tile: piece p = 64 t + lane of [32 rows][13 pieces] (416 = 6.5 x 64), and the
+  // row's last two bytes (d) by lanes 0..31
+  size_t woff[7];
+  u32 wdst[7];
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b) val[2 * a + b] = fmaf(tot[4 * a + 2 * b + 1], 0.00048828125f, tot[4 * a + 2 * b]);
-  if (kparts == 1u) {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
-        if (row_ok && token < m) c[static_cast<size_t>(token) * n + row] = val[2 * a + b];
-      }
-    return;
+  for (int t = 0; t < 7; ++t) {
+    const u32 p = min(64u * t + lane, 415u);
+    const u32 r = p / 13u, cc = p - 13u * r;
+    woff[t] = static_cast<size_t>(min(strip * 32u + r, n - 1u)) * row_bytes + 16u * cc;
+    wdst[t] = r * kQ6RowStride + 16u * cc;
   }
-  // several parts of K: publish this part, the last arrival adds them up.  The parts cross workgroups (and XCDs):
-  // 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side by side:
-  //   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
-  const u32 strips = groups * waves;
-  const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      partial, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
-  auto slot_of = [&](u32 pt) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
-  __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[0]), __float_as_uint(val[1]), __float_as_uint(val[2]), __float_as_uint(val[3])},
-                                         part_rsrc, slot_of(part), 0, 16);
-  const bool upper = tile * kTokensPerTile + 8u < m;      // tokens 8..15 of the tile exist (val[4..7])
-  if (upper)
-    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[4]), __float_as_uint(val[5]), __float_as_uint(val[6]), __float_as_uint(val[7])},
-                                           part_rsrc, slot_of(part) + 16, 0, 16);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
-  asm volatile("s_barrier" ::: "memory");
-  if (threadIdx.x == 0u) {
-    const u32 old = __hip_atomic_fetch_add(counters + group * tiles + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(lds_flag), "v"(old) : "memory");
-  }
-  asm volatile("s_barrier" ::: "memory");
-  u32 old;
-  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(lds_flag) : "memory");
-  if (old == kparts - 1u && threadIdx.x == 0u)      // ready for the next product on this stream
-    __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (old != kparts - 1u || !row_ok) return;
-  float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // eight parts in flight, added in part order
-    u32x4 lo[8], hi[8];
+  const size_t doff = static_cast<size_t>(min(strip * 32u + col, n - 1u)) * row_bytes + 208u;
+  const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * kQ6TileBytes;
+  const u32 lds_flag = lds_base + 2u * kXpStageBytes + waves * kQ6TileBytes;
+  const u32 nthreads = blockDim.x;
+  const float* asrc[CHUNKS];
+  u32 ctoken[CHUNKS], cpos[CHUNKS];
+  bool live[CHUNKS];
 #pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp) {
-      const u32 pt = min(p0 + pp, kparts - 1u);
-      lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
-      hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
+  for (int i = 0; i < CHUNKS; ++i) {
+    const u32 idx = threadIdx.x + i * nthreads;
+    ctoken[i] = (idx >> 5) & 15u;
+    cpos[i] = idx & 31u;
+    const u32 token = tile * kTokensPerTile + ctoken[i];
+    asrc[i] = a + static_cast<size_t>(min(token, m - 1u)) * (static_cast<size_t>(nsb) * 256u) + 8u * cpos[i];
+    live[i] = token < m;
+  }
+
+  // The loads of this kernel are ordinary ones and the compiler places the waits: values that stay in registers from
+  // one super-block to the next and meet at the joins of the loop are copied where the compiler sees fit, which it may
+  // only do with data that has arrived if it knows the load.  (The LDS side is written out by hand as in the Q4_K kernel.)
+  u32x4 wn[7];                         // the next super-block's weight tile on its way to LDS
+  u32 wd;
+  auto load_w = [&](u32 s) {
+    const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * 210u;
+#pragma unroll
+    for (int t = 0; t < 7; ++t) wn[t] = load128_a2(wsrc + woff[t]);
+    wd = load16_a2(wsrc + doff);
+  };
+  auto store_w = [&]() {
+#pragma unroll
+    for (int t = 0; t < 6; ++t) asm volatile("ds_write_b128 %0, %1" ::"v"(lds_w + wdst[t]), "v"(wn[t]) : "memory");
+    if (lane < 32u) {
+      asm volatile("ds_write_b128 %0, %1" ::"v"(lds_w + wdst[6]), "v"(wn[6]) : "memory");
+      asm volatile("ds_write_b16 %0, %1" ::"v"(lds_w + col * kQ6RowStride + 208u), "v"(wd) : "memory");
     }
+  };
+  f32x4 an[CHUNKS][2];
+  auto load_a = [&](u32 s) {
 #pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp)
-      if (p0 + pp < kparts) {
-        r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
-        r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
+    for (int i = 0; i < CHUNKS; ++i) {
+      const f32x4* src = reinterpret_cast<const f32x4*>(asrc[i] + static_cast<size_t>(sb0 + s) * 256u);
+      an[i][0] = src[0];
+      an[i][1] = src[1];
+    }
+  };
+  auto convert = [&](u32 s) {
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i)
+      convert_chunk<false>(live[i] ? an[i][0] : zero4, live[i] ? an[i][1] : zero4, ctoken[i], cpos[i], lds_xp + (s & 1u) * kXpStageBytes);
+  };
+
+  f32x16 tot;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) tot[v] = 0.0f;
+  u32 xq[16];                                    // where this lane finds its token operands of page Q (stage 0)
+#pragma unroll
+  for (u32 q = 0; q < 16; ++q) xq[q] = lds_xp + ((lane ^ (2u * q)) << 4);
+
+  // One super-block.  NEXT / NEXT2: super-blocks s+1 / s+2 exist (compile-time, so that every load is unconditional
+  // where it stands: the loop below is peeled at its end).
+  auto step = [&](u32 s, auto next_c, auto next2_c) {
+    constexpr bool NEXT = decltype(next_c)::value, NEXT2 = decltype(next2_c)::value;
+    // tile s is in LDS (this wave wrote it), the token operands of s are written by everybody
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    const u32 slot = s & 1u;
+    const u32 wt = lds_w + col * kQ6RowStride;
+    const u32 fl = lds_xp + slot * kXpStageBytes + kXpMainBytes + kXpSumBytes + g * 8u;
+    u32x4 l0, l1, l2, l3, h0, h1;
+    u32x2 scv, f01, f23, f45, f67;
+    u32 dv;
+    lds_read128<0>(l0, wt + g * 64u);
+    lds_read128<16>(l1, wt + g * 64u);
+    lds_read128<32>(l2, wt + g * 64u);
+    lds_read128<48>(l3, wt + g * 64u);
+    lds_read128<128>(h0, wt + g * 32u);
+    lds_read128<144>(h1, wt + g * 32u);
+    lds_read64<192>(scv, wt + g * 8u);
+    asm volatile("ds_read_u16 %0, %1 offset:208" : "=&v"(dv) : "v"(wt) : "memory");
+    lds_read64<0>(f01, fl);          // 2^(E+14) of the tokens 4a + 2g + {0, 1}, a = 0..3
+    lds_read64<16>(f23, fl);
+    lds_read64<32>(f45, fl);
+    lds_read64<48>(f67, fl);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(l0), "+v"(l1), "+v"(l2), "+v"(l3), "+v"(h0), "+v"(h1), "+v"(scv), "+v"(dv)::"memory");
+    asm volatile("" : "+v"(f01), "+v"(f23), "+v"(f45), "+v"(f67));
+    if constexpr (NEXT) convert(s + 1u);     // into the stage that was read two super-blocks ago
+    if constexpr (NEXT2) load_a(s + 2u);
+    const u32 ql[16] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w, l2.x, l2.y, l2.z, l2.w, l3.x, l3.y, l3.z, l3.w};
+    const u32 qh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+    const float d = half_bits_to_f32(dv);
+    // this lane's eight int8 scales (sub-blocks 8g .. 8g+7) as the factors and addends of the two multiply-adds, each
+    // doubled into both halves of a word
+    h16x2 sn[8], an8[8], sq[8], aq3[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const u32 word = e < 4 ? scv.x : scv.y;
+      const int sv = static_cast<int>(static_cast<int8_t>((word >> (8 * (e & 3))) & 0xFFu));
+      const _Float16 sf = static_cast<_Float16>(static_cast<short>(sv));
+      const _Float16 f_n = sf * static_cast<_Float16>(64.0f), a_n = sf * static_cast<_Float16>(-0.00048828125f);      // -8 * 2^-14
+      const _Float16 f_q = sf * static_cast<_Float16>(128.0f), a_q = sf * static_cast<_Float16>(-0.00018310546875f);  // -3 * 2^-14
+      sn[e] = h16x2{f_n, f_n};
+      an8[e] = h16x2{a_n, a_n};
+      sq[e] = h16x2{f_q, f_q};
+      aq3[e] = h16x2{a_q, a_q};
+    }
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    f32x16 acc_n = zero, acc_q = zero;
+#pragma unroll
+    for (int q0 = 0; q0 < 16; q0 += 4) {         // four token pages per round of operand reads, two products a page
+      u32x4 a0, a1, a2, a3;
+      const u32 xs = slot * kXpStageBytes;
+      switch (q0) {
+        case 0: lds_read128<0 * 1024>(a0, xq[0] + xs); lds_read128<1 * 1024>(a1, xq[1] + xs); lds_read128<2 * 1024>(a2, xq[2] + xs); lds_read128<3 * 1024>(a3, xq[3] + xs); break;
+        case 4: lds_read128<4 * 1024>(a0, xq[4] + xs); lds_read128<5 * 1024>(a1, xq[5] + xs); lds_read128<6 * 1024>(a2, xq[6] + xs); lds_read128<7 * 1024>(a3, xq[7] + xs); break;
+        case 8: lds_read128<8 * 1024>(a0, xq[8] + xs); lds_read128<9 * 1024>(a1, xq[9] + xs); lds_read128<10 * 1024>(a2, xq[10] + xs); lds_read128<11 * 1024>(a3, xq[11] + xs); break;
+        default: lds_read128<12 * 1024>(a0, xq[12] + xs); lds_read128<13 * 1024>(a1, xq[13] + xs); lds_read128<14 * 1024>(a2, xq[14] + xs); lds_read128<15 * 1024>(a3, xq[15] + xs); break;
       }
-  }
+      const u32x4* aq[4] = {&a0, &a1, &a2, &a3};
+      u32 bn[4][4], bq[4][4];
 #pragma unroll
-  for (int t = 0; t < 8; ++t) {
-    const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
-    if (token < m) c[static_cast<size_t>(token) * n + row] = r[t];
+      for (int i = 0; i < 4; ++i) {
+        const int Q = q0 + i, U = Q >> 1, H = Q & 1, hi_nib = U >> 2, gq = 2 * (U >> 2) + H;
+        const int e = 2 * gq + ((U & 3) >> 1);
+        const u32 t0 = ql[8 * H + 2 * (U & 3)], t1 = ql[8 * H + 2 * (U & 3) + 1];
+        // nibbles to bits 4..7 of their 16-bit lanes: bytes 0 and 2, then bytes 1 and 3
+        const u32 n00 = hi_nib ? t0 : t0 << 4, n01 = hi_nib ? t0 >> 8 : t0 >> 4;
+        const u32 n10 = hi_nib ? t1 : t1 << 4, n11 = hi_nib ? t1 >> 8 : t1 >> 4;
+        bn[i][0] = __builtin_bit_cast(u32, pk_fma_h2(n00 & 0x00F000F0u, sn[e], an8[e]));
+        bn[i][1] = __builtin_bit_cast(u32, pk_fma_h2(n01 & 0x00F000F0u, sn[e], an8[e]));
+        bn[i][2] = __builtin_bit_cast(u32, pk_fma_h2(n10 & 0x00F000F0u, sn[e], an8[e]));
+        bn[i][3] = __builtin_bit_cast(u32, pk_fma_h2(n11 & 0x00F000F0u, sn[e], an8[e]));
+        // field gq of the qh bytes to bits 4..5: shift by 4 - 2 gq (bytes 0 and 2), by -4 - 2 gq (bytes 1 and 3)
+        const u32 c0 = qh[2 * (U & 3)], c1 = qh[2 * (U & 3) + 1];
+        const u32 f00 = gq == 0 ? c0 << 4 : gq == 1 ? c0 << 2 : gq == 2 ? c0 : c0 >> 2, f01v = c0 >> (4 + 2 * gq);
+        const u32 f10 = gq == 0 ? c1 << 4 : gq == 1 ? c1 << 2 : gq == 2 ? c1 : c1 >> 2, f11 = c1 >> (4 + 2 * gq);
+        bq[i][0] = __builtin_bit_cast(u32, pk_fma_h2(f00 & 0x00300030u, sq[e], aq3[e]));
+        bq[i][1] = __builtin_bit_cast(u32, pk_fma_h2(f01v & 0x00300030u, sq[e], aq3[e]));
+        bq[i][2] = __builtin_bit_cast(u32, pk_fma_h2(f10 & 0x00300030u, sq[e], aq3[e]));
+        bq[i][3] = __builtin_bit_cast(u32, pk_fma_h2(f11 & 0x00300030u, sq[e], aq3[e]));
+      }
+      lds_wait4(a0, a1, a2, a3);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u32x4 bnv = {bn[i][0], bn[i][1], bn[i][2], bn[i][3]}, bqv = {bq[i][0], bq[i][1], bq[i][2], bq[i][3]};
+        acc_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[i]), __builtin_bit_cast(h16x8, bnv), acc_n, 0, 0, 0);
+        acc_q = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[i]), __builtin_bit_cast(h16x8, bqv), acc_q, 0, 0, 0);
+      }
+    }
+    // the next tile's registers to LDS: this wave is done reading the current one
+    if constexpr (NEXT) store_w();
+    if constexpr (NEXT2) load_w(s + 2u);
+    const float fac[8] = {__uint_as_float(f01.x), __uint_as_float(f01.y), __uint_as_float(f23.x), __uint_as_float(f23.y),
+                          __uint_as_float(f45.x), __uint_as_float(f45.y), __uint_as_float(f67.x), __uint_as_float(f67.y)};
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float fd = fac[t] * d;
+#pragma unroll
+      for (int pc = 0; pc < 2; ++pc) {
+        const int v = 2 * t + pc;
+        tot[v] = fmaf(fd, fmaf(8.0f, acc_q[v], acc_n[v]), tot[v]);
+      }
+    }
+  };
+  using std::true_type;
+  using std::false_type;
+  load_a(0);
+  load_w(0);
+  __builtin_amdgcn_sched_barrier(0);   // both sets of loads on their way before the conversion waits for the first
+  convert(0);
+  store_w();
+  if (ns == 1u) {
+    step(0u, false_type{}, false_type{});
+  } else {
+    load_a(1);
+    load_w(1);
+    u32 s = 0;
+    for (; s + 2u < ns; ++s) step(s, true_type{}, true_type{});
+    step(s, true_type{}, false_type{});
+    step(s + 1u, false_type{}, false_type{});
   }
+  finish_tile(tot, c, partial, counters, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
 }
 
 }  // namespace gemm_f16

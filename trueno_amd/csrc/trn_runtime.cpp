@@ -76,7 +76,7 @@ struct DeviceKernels {
   hipFunction_t copy_u128 = nullptr, read_u128 = nullptr;
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
-  hipFunction_t gemm_f16[2][2] = {};   // [Q4_K, Q5_K][4 or 8 strips per workgroup]
+  hipFunction_t gemm_f16[NFMT][2] = {};   // [format][4 or 8 strips per workgroup]
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
@@ -157,6 +157,8 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.gemm_f16[0][1], "q4k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[1][0], "q5k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[1][1], "q5k_gemm_f16_w8")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[2][0], "q6k_gemm_f16_w4")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16[2][1], "q6k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -373,9 +375,12 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
                               uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
   const uint32_t kGemmWTileBytes = 32u * kSbBytes[f];
+  // Q6_K: one weight tile per wave, rows 240 bytes apart (q6k_lds_bytes of the kernel's header)
+  const uint32_t kGemmQ6TileBytes = 32u * 240u;
   // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
   const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
-  const uint32_t lds = 2u * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
+  const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
+                                : 2u * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
   const uint32_t groups = (n + 32u * waves - 1u) / (32u * waves);
   // cut K so that the workgroups are about as many as the CUs
   const uint64_t units = uint64_t(groups) * tiles;
@@ -402,24 +407,24 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
   uint32_t nsb_arg = nsb, ksb_arg = ksb, kparts_arg = kparts, groups_arg = groups, tiles_arg = tiles;
   void* margs[] = {&a, &w, &c, &part, &cnt, &m, &n, &nsb_arg, &ksb_arg, &kparts_arg, &groups_arg, &tiles_arg};
-  return hipModuleLaunchKernel(d->gemm_f16[f == Q5K][waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
+  return hipModuleLaunchKernel(d->gemm_f16[f][waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
-// does the matrix-core form take this product?  (Q4_K and Q5_K)
-bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
-  return m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, 16) && aligned(c, 4) &&
+// does the matrix-core form take this product?  (weights 16-byte aligned; Q6_K, whose blocks are 210 bytes, 2-byte aligned)
+bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k, Fmt f = Q4K) {
+  return m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, f == Q6K ? 2 : 16) && aligned(c, 4) &&
          uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u;   // its arrival counters
 }
 
 // A few tokens against a small matrix are faster through the GEMV engine, one pass per token with the weights of the
 // second and later passes coming from the caches, than through the matrix-core kernel with its start-up and its sum
 // over the parts of K.  Times in microseconds fitted to measurements on MI355X (MB = weight bytes / 1e6):
-//   engine: 3.9 + MB / 5.7 for the first token, MB / 7 + 0.4 for each further one (one slab of columns only; with
+//   engine: 3.9 + MB / 5.7 for the first token, MB / 5.8 + 0.15 for each further one (one slab of columns only; with
 //   k > 4096 a further pass costs as much as the first); matrix cores: 12 + MB / 9.4 for up to 16 tokens.
 bool gemm_few_tokens_by_engine(Fmt f, uint32_t m, uint32_t n, uint32_t k) {
   if (m > 8u || k > 4096u) return false;
   const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
-  return 3.9 + mb / 5.7 + (m - 1u) * (mb / 7.0 + 0.4) < 12.0 + mb / 9.4;
+  return 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15) < 12.0 + mb / 9.4;
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
@@ -430,7 +435,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
-  if (!is_gemv && (f == Q4K || f == Q5K) && q4k_gemm_f16_ok(a, w, c, m, n, k) &&
+  if (!is_gemv && q4k_gemm_f16_ok(a, w, c, m, n, k, f) &&
       (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || !gemm_few_tokens_by_engine(f, m, n, k)))
     return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
