@@ -176,16 +176,18 @@ __device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, 
 __device__ __forceinline__ h16x2 pk_mul_h2(u32 bits, h16x2 s) { return as_h16x2(bits) * s; }
 __device__ __forceinline__ h16x2 pk_fma_h2(u32 bits, h16x2 s, h16x2 add) { return __builtin_elementwise_fma(as_h16x2(bits), s, add); }
 
+constexpr u32 kCounterBytes = 1u << 16;        // arrival counters at the front of the workspace, the partial sums behind them
+
 // What the kernels do with a finished tile.  lane l, tot registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row
 // strip*32 + col.  With one part of K the result is stored; otherwise the part is published and the workgroup that
-// arrives last at the (group, tile) counter adds the parts in part order and puts the counter back to zero.
-__device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict__ c, float* __restrict__ partial, u32* __restrict__ counters,
+// arrives last at the (group, tile) counter adds the parts in part order - the sum does not depend on who is last -
+// and puts the counter back to zero.  (A counter per strip, each wave on its own without the two barriers, was
+// measured 0.5-1 us slower: eight times as many atomic operations on neighbouring addresses.)
+__device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict__ c, uint8_t* __restrict__ ws,
                                             u32 m, u32 n, u32 kparts, u32 groups, u32 tiles, u32 waves, u32 group, u32 part, u32 tile,
                                             u32 strip, u32 col, u32 g, u32 lane, u32 lds_flag) {
-  // lane l, registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row strip*32 + col
   const u32 row = strip * 32u + col;
   const bool row_ok = row < n;
-  const u32 tokens_pad = tiles * kTokensPerTile;
   float val[8];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
@@ -201,12 +203,12 @@ __device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict
       }
     return;
   }
-  // several parts of K: publish this part, the last arrival adds them up.  The parts cross workgroups (and XCDs):
-  // 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side by side:
-  //   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
+  // The parts cross workgroups (and XCDs): 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side
+  // by side:   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
+  u32* counters = reinterpret_cast<u32*>(ws);
   const u32 strips = groups * waves;
   const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      partial, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
+      ws + kCounterBytes, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
   auto slot_of = [&](u32 pt) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
   __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[0]), __float_as_uint(val[1]), __float_as_uint(val[2]), __float_as_uint(val[3])},
                                          part_rsrc, slot_of(part), 0, 16);
@@ -227,27 +229,46 @@ __device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict
     __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (old != kparts - 1u || !row_ok) return;
   float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  for (u32 p0 = 0; p0 < kparts; p0 += 8u) {          // eight parts in flight, added in part order
-    u32x4 lo[8], hi[8];
+  // all parts in flight at once when they are at most sixteen (a round trip to memory each time otherwise), added in
+  // part order; no more loads than there are parts to the next power of two
+  auto add_parts = [&](auto width) {
+    constexpr u32 W = decltype(width)::value;
+    for (u32 p0 = 0; p0 < kparts; p0 += W) {
+      u32x4 lo[W], hi[W];
 #pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp) {
-      const u32 pt = min(p0 + pp, kparts - 1u);
-      lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
-      hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
-    }
-#pragma unroll
-    for (u32 pp = 0; pp < 8; ++pp)
-      if (p0 + pp < kparts) {
-        r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
-        r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
+      for (u32 pp = 0; pp < W; ++pp) {
+        const u32 pt = min(p0 + pp, kparts - 1u);
+        lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
+        hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
       }
-  }
+#pragma unroll
+      for (u32 pp = 0; pp < W; ++pp)
+        if (p0 + pp < kparts) {
+          r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
+          r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
+        }
+    }
+  };
+  if (kparts <= 2u) add_parts(std::integral_constant<u32, 2>{});
+  else if (kparts <= 4u) add_parts(std::integral_constant<u32, 4>{});
+  else if (kparts <= 8u) add_parts(std::integral_constant<u32, 8>{});
+  else add_parts(std::integral_constant<u32, 16>{});
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
     if (token < m) c[static_cast<size_t>(token) * n + row] = r[t];
   }
 }
+
+// What every kernel of this file takes: the operands, the workspace (counters, then partial sums), the shape and
+// the cut - geom = ksb | kparts << 16 | groups << 32 | tiles << 48 - in eight arguments, which the hardware hands
+// over in registers at the start of a wave (kernel-argument preload), so that nothing is read before the first loads.
+struct Geometry {
+  u32 ksb, kparts, groups, tiles;
+  __device__ explicit Geometry(uint64_t geom)
+      : ksb(static_cast<u32>(geom) & 0xFFFFu), kparts(static_cast<u32>(geom >> 16) & 0xFFFFu),
+        groups(static_cast<u32>(geom >> 32) & 0xFFFFu), tiles(static_cast<u32>(geom >> 48)) {}
+};
 
 // Main kernel.  Workgroup id -> (unit, token tile) with the token tiles of a unit 8 ids apart (same XCD, so the
 // weights they share meet in that XCD's L2); unit -> (group of 8 strips, part of K).  With one part the result
@@ -256,9 +277,10 @@ __device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict
 // puts the counter back to zero (the counters start at zero when the workspace is allocated).
 //   dynamic LDS = kLdsBytes
 template <int FMT, int CHUNKS>     // CHUNKS: chunks of A a thread converts per super-block, 512 / threads
-__device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
-                                         u32* __restrict__ counters, u32 m, u32 n, u32 nsb, u32 ksb, u32 kparts,
-                                         u32 groups, u32 tiles, u32 lds_base) {
+__device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, uint8_t* __restrict__ ws,
+                                         u32 m, u32 n, u32 nsb, uint64_t geom, u32 lds_base) {
+  const Geometry cut(geom);
+  const u32 ksb = cut.ksb, kparts = cut.kparts, groups = cut.groups, tiles = cut.tiles;
   const u32 lane = threadIdx.x & 63u;
   const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
   const u32 id = blockIdx.x;
@@ -266,7 +288,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   if (unit >= groups * kparts) return;
   const u32 group = unit / kparts, part = unit - group * kparts;
   const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
-  const u32 waves = blockDim.x >> 6;
+  constexpr u32 waves = 8u / CHUNKS;      // the kernels are launched with 512 / CHUNKS threads
   const u32 strip = group * waves + wave;
   const u32 col = lane & 31u, g = lane >> 5;
   using T = WTile<FMT>;
@@ -285,7 +307,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * (2u * kWStageBytes);
   const u32 lds_flag = lds_base + 2u * kXpStageBytes + 2u * waves * kWStageBytes;
   // the chunks of A this thread converts per super-block: 512 chunks of 8 elements (16 tokens x 32)
-  const u32 nthreads = blockDim.x;
+  constexpr u32 nthreads = 512u / CHUNKS;
   const float* asrc[CHUNKS];
   u32 ctoken[CHUNKS], cpos[CHUNKS];
   bool live[CHUNKS];
@@ -460,7 +482,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     }
   }
 
-  finish_tile(tot, c, partial, counters, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
+  finish_tile(tot, c, ws, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
 }
 
 
@@ -486,9 +508,10 @@ constexpr u32 kQ6TileBytes = 32u * kQ6RowStride;
 __host__ __device__ constexpr u32 q6k_lds_bytes(u32 waves) { return 2u * kXpStageBytes + waves * kQ6TileBytes + 16u; }
 
 template <int CHUNKS>
-__device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, float* __restrict__ partial,
-                                         u32* __restrict__ counters, u32 m, u32 n, u32 nsb, u32 ksb, u32 kparts,
-                                         u32 groups, u32 tiles, u32 lds_base) {
+__device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, uint8_t* __restrict__ ws,
+                                         u32 m, u32 n, u32 nsb, uint64_t geom, u32 lds_base) {
+  const Geometry cut(geom);
+  const u32 ksb = cut.ksb, kparts = cut.kparts, groups = cut.groups, tiles = cut.tiles;
   const u32 lane = threadIdx.x & 63u;
   const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
   const u32 id = blockIdx.x;
@@ -496,7 +519,7 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
   if (unit >= groups * kparts) return;
   const u32 group = unit / kparts, part = unit - group * kparts;
   const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
-  const u32 waves = blockDim.x >> 6;
+  constexpr u32 waves = 8u / CHUNKS;      // the kernels are launched with 512 / CHUNKS threads
   const u32 strip = group * waves + wave;
   const u32 col = lane & 31u, g = lane >> 5;
   const size_t row_bytes = static_cast<size_t>(nsb) * 210u;
@@ -515,7 +538,7 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
   const size_t doff = static_cast<size_t>(min(strip * 32u + col, n - 1u)) * row_bytes + 208u;
   const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * kQ6TileBytes;
   const u32 lds_flag = lds_base + 2u * kXpStageBytes + waves * kQ6TileBytes;
-  const u32 nthreads = blockDim.x;
+  constexpr u32 nthreads = 512u / CHUNKS;
   const float* asrc[CHUNKS];
   u32 ctoken[CHUNKS], cpos[CHUNKS];
   bool live[CHUNKS];
@@ -692,7 +715,7 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
     step(s, true_type{}, false_type{});
     step(s + 1u, false_type{}, false_type{});
   }
-  finish_tile(tot, c, partial, counters, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
+  finish_tile(tot, c, ws, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
 }
 
 }  // namespace gemm_f16

@@ -272,32 +272,22 @@ KQ_GEMM_KERNELS(q4k, FMT_Q4K)
 KQ_GEMM_KERNELS(q5k, FMT_Q5K)
 KQ_GEMM_KERNELS(q6k, FMT_Q6K)
 
-// Matrix-core form of the Q4_K and Q5_K GEMM for m >= 2 (kquant_gemm_f16.hip.h).
-#define KQ_GEMM_F16(name, threads, FMT)                                                                                 \
+// Matrix-core form of the k-quant GEMM for m >= 2 (kquant_gemm_f16.hip.h; the arguments: Geometry there).
+#define KQ_GEMM_F16(name, threads, BODY)                                                                                \
   extern "C" __global__ void __launch_bounds__(threads)                                                                  \
-  name(const float* a, const uint8_t* w, float* c, float* partial, u32* counters, u32 m, u32 n, u32 nsb, u32 ksb,        \
-       u32 kparts, u32 groups, u32 tiles) {                                                                              \
+  name(const float* a, const uint8_t* w, float* c, uint8_t* ws, u32 m, u32 n, u32 nsb, uint64_t geom) {                  \
     extern __shared__ uint8_t gemm_lds[];                                                                                \
     const u32 lds_base =                                                                                                 \
         static_cast<u32>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) uint8_t*)gemm_lds));         \
-    gemm_f16::kq_body<FMT, 512 / threads>(a, w, c, partial, counters, m, n, nsb, ksb, kparts, groups, tiles, lds_base); \
+    gemm_f16::BODY(a, w, c, ws, m, n, nsb, geom, lds_base);                                                              \
   }
-KQ_GEMM_F16(q4k_gemm_f16_w8, 512, FMT_Q4K)
-KQ_GEMM_F16(q4k_gemm_f16_w4, 256, FMT_Q4K)
-KQ_GEMM_F16(q5k_gemm_f16_w8, 512, FMT_Q5K)
-KQ_GEMM_F16(q5k_gemm_f16_w4, 256, FMT_Q5K)
-// Q6_K on the matrix cores (q6k_body of kquant_gemm_f16.hip.h): same arguments.
-#define KQ_GEMM_F16_Q6K(name, threads)                                                                                  \
-  extern "C" __global__ void __launch_bounds__(threads)                                                                  \
-  name(const float* a, const uint8_t* w, float* c, float* partial, u32* counters, u32 m, u32 n, u32 nsb, u32 ksb,        \
-       u32 kparts, u32 groups, u32 tiles) {                                                                              \
-    extern __shared__ uint8_t gemm_lds[];                                                                                \
-    const u32 lds_base =                                                                                                 \
-        static_cast<u32>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) uint8_t*)gemm_lds));         \
-    gemm_f16::q6k_body<512 / threads>(a, w, c, partial, counters, m, n, nsb, ksb, kparts, groups, tiles, lds_base);      \
-  }
-KQ_GEMM_F16_Q6K(q6k_gemm_f16_w8, 512)
-KQ_GEMM_F16_Q6K(q6k_gemm_f16_w4, 256)
+#define KQ_COMMA ,
+KQ_GEMM_F16(q4k_gemm_f16_w8, 512, kq_body<FMT_Q4K KQ_COMMA 1>)
+KQ_GEMM_F16(q4k_gemm_f16_w4, 256, kq_body<FMT_Q4K KQ_COMMA 2>)
+KQ_GEMM_F16(q5k_gemm_f16_w8, 512, kq_body<FMT_Q5K KQ_COMMA 1>)
+KQ_GEMM_F16(q5k_gemm_f16_w4, 256, kq_body<FMT_Q5K KQ_COMMA 2>)
+KQ_GEMM_F16(q6k_gemm_f16_w8, 512, q6k_body<1>)
+KQ_GEMM_F16(q6k_gemm_f16_w4, 256, q6k_body<2>)
 
 // Legacy "simplified" Q4_K (trueno-gpu/src/kernels/quantize.rs:151-336, kernel name q4k_gemm_fused): blocks of 32
 // values in 18 bytes - f16 scale at 0, 16 bytes of nibbles at 2, value i in byte i/2 (low nibble for even i);

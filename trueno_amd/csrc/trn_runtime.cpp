@@ -389,7 +389,8 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   const uint32_t ksb = (nsb + kparts - 1u) / kparts;
   kparts = (nsb + ksb - 1u) / ksb;
   auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
-  const size_t cnt_bytes = up(size_t(groups) * tiles * 4u);
+  // with several parts of K: one arrival counter per (group of strips, token tile)
+  const size_t cnt_bytes = kparts > 1u ? size_t(groups) * tiles * 4u : 0u;
   // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
   const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * groups * waves * 2048u) : 0u;
   // the counters sit at the front of a region that only grows, so a larger product finds zeros there too (the
@@ -403,17 +404,19 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
     hipError_t e = acquire_scratch(g_gemm_ws, d, stream, need, cnt_cap, &cnt);
     if (e != hipSuccess) return e;
   }
-  uint64_t part = cnt + cnt_cap;
   const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
-  uint32_t nsb_arg = nsb, ksb_arg = ksb, kparts_arg = kparts, groups_arg = groups, tiles_arg = tiles;
-  void* margs[] = {&a, &w, &c, &part, &cnt, &m, &n, &nsb_arg, &ksb_arg, &kparts_arg, &groups_arg, &tiles_arg};
+  if (ksb > 0xFFFFu || groups > 0xFFFFu || tiles > 0xFFFFu || padded * tiles > 0x7FFFFFFFu) return hipErrorInvalidValue;
+  uint32_t nsb_arg = nsb;
+  uint64_t geom = uint64_t(ksb) | uint64_t(kparts) << 16 | uint64_t(groups) << 32 | uint64_t(tiles) << 48;
+  void* margs[] = {&a, &w, &c, &cnt, &m, &n, &nsb_arg, &geom};
   return hipModuleLaunchKernel(d->gemm_f16[f][waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
 // does the matrix-core form take this product?  (weights 16-byte aligned; Q6_K, whose blocks are 210 bytes, 2-byte aligned)
 bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k, Fmt f = Q4K) {
   return m >= 2 && k != 0 && !g_tune_gemm_mfma_off && aligned(a, 16) && aligned(w, f == Q6K ? 2 : 16) && aligned(c, 4) &&
-         uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 16384u;   // its arrival counters
+         k / 256u <= 0xFFFFu && (n + 127u) / 128u <= 0xFFFFu && (m + 15u) / 16u <= 0xFFFFu &&      // 16-bit fields of its geometry
+         uint64_t((n + 127u) / 128u) * ((m + 15u) / 16u) <= 0x0FFFFFFFu;                            // its grid
 }
 
 // A few tokens against a small matrix are faster through the GEMV engine, one pass per token with the weights of the
