@@ -107,6 +107,41 @@ def test_gemm_matrix_core_form_ragged(gpu, fmt, n, k, m):
     assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
 
 
+@pytest.mark.parametrize("m", (17, 33, 40, 64))
+@pytest.mark.parametrize("fmt", ("q4k", "q5k"))
+def test_gemm_two_token_tiles_per_workgroup(gpu, fmt, m):
+    """The kernels that take two tiles of 16 tokens per workgroup, forced on a small product: odd numbers of tiles
+    (the second tile of the last pair does not exist), K in one part and in several, the same bits on every run;
+    and one tile per workgroup gives the same bits for the same cut of K (a tile's sums do not depend on its
+    company)."""
+    n, k = 300, 1536
+    buf, a = kq.gen_matrix(fmt, 70 + m, n, k), kq.gen_x(80 + m, m, k)
+    c64 = _c64(fmt, buf, a, n, k)
+    try:
+        for parts in (1, 3):
+            _tune("gemm_k_parts", parts)
+            _tune("gemm_tiles", 2)
+            two = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+            assert kq.rel_l2(two, c64) <= TOL
+            again = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+            assert np.array_equal(again.view(np.uint32), two.view(np.uint32)), parts
+            _tune("gemm_tiles", 1)
+            one = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+            assert np.array_equal(one.view(np.uint32), two.view(np.uint32)), parts
+    finally:
+        _tune("gemm_k_parts", 0)
+        _tune("gemm_tiles", 0)
+
+
+@pytest.mark.parametrize("fmt", ("q4k", "q5k"))
+def test_gemm_many_tokens(gpu, fmt):
+    """512 tokens against 4096 x 2048: enough workgroups that the library itself takes two tiles per workgroup."""
+    n, k, m = 4096, 2048, 512
+    buf, a = kq.gen_matrix(fmt, 77, n, k), kq.gen_x(78, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
+
+
 @pytest.mark.parametrize("fmt", MFMA_FORMATS)
 def test_gemm_parts_of_k(gpu, fmt):
     """However K is cut into parts the result stays within tolerance, and the same cut gives the same bits on

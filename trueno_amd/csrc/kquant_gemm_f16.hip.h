@@ -62,7 +62,7 @@ template <int FMT> struct WTile;
 template <> struct WTile<FMT_Q4K> { static constexpr u32 SB = 144, PIECES = 9, DMA = 5, BYTES = 32 * 144; };
 template <> struct WTile<FMT_Q5K> { static constexpr u32 SB = 176, PIECES = 11, DMA = 6, BYTES = 32 * 176; };
 // dynamic LDS: two stages of token operands, two weight tiles per wave, one word for the arrival order
-__host__ __device__ constexpr u32 lds_bytes(u32 waves, u32 tile_bytes) { return 2u * kXpStageBytes + 2u * waves * tile_bytes + 16u; }
+__host__ __device__ constexpr u32 lds_bytes(u32 waves, u32 tile_bytes, u32 nt) { return 2u * nt * kXpStageBytes + 2u * waves * tile_bytes + 16u; }
 
 __device__ __forceinline__ u32 wave_max_u32(u32 v) {
   v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true)));
@@ -178,29 +178,35 @@ __device__ __forceinline__ h16x2 pk_fma_h2(u32 bits, h16x2 s, h16x2 add) { retur
 
 constexpr u32 kCounterBytes = 1u << 16;        // arrival counters at the front of the workspace, the partial sums behind them
 
-// What the kernels do with a finished tile.  lane l, tot registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row
-// strip*32 + col.  With one part of K the result is stored; otherwise the part is published and the workgroup that
-// arrives last at the (group, tile) counter adds the parts in part order - the sum does not depend on who is last -
-// and puts the counter back to zero.  (A counter per strip, each wave on its own without the two barriers, was
-// measured 0.5-1 us slower: eight times as many atomic operations on neighbouring addresses.)
-__device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict__ c, uint8_t* __restrict__ ws,
-                                            u32 m, u32 n, u32 kparts, u32 groups, u32 tiles, u32 waves, u32 group, u32 part, u32 tile,
-                                            u32 strip, u32 col, u32 g, u32 lane, u32 lds_flag) {
+// What the kernels do with the finished tiles of a workgroup (NT token tiles of 16: tiles tg*NT .. tg*NT + NT - 1).
+// lane l, tot registers 4a + 2b + piece: token 4a + 2g + b of the tile, W row strip*32 + col.  With one part of K the
+// results are stored; otherwise the part is published and the workgroup that arrives last at the (group, tile group)
+// counter adds the parts in part order - the sum does not depend on who is last - and puts the counter back to zero.
+// (A counter per strip, each wave on its own without the two barriers, was measured 0.5-1 us slower: eight times as
+// many atomic operations on neighbouring addresses.)
+template <int NT>
+__device__ __forceinline__ void finish_tiles(const f32x16 (&tot)[NT], float* __restrict__ c, uint8_t* __restrict__ ws,
+                                             u32 m, u32 n, u32 kparts, u32 groups, u32 tiles, u32 tgroups, u32 waves, u32 group, u32 part,
+                                             u32 tg, u32 strip, u32 col, u32 g, u32 lane, u32 lds_flag) {
   const u32 row = strip * 32u + col;
   const bool row_ok = row < n;
-  float val[8];
+  float val[NT][8];
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b) val[2 * a + b] = fmaf(tot[4 * a + 2 * b + 1], 0.00048828125f, tot[4 * a + 2 * b]);
-  if (kparts == 1u) {
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const u32 token = tile * kTokensPerTile + 4u * a + 2u * g + b;
-        if (row_ok && token < m) c[static_cast<size_t>(token) * n + row] = val[2 * a + b];
-      }
+      for (int b = 0; b < 2; ++b) val[t][2 * a + b] = fmaf(tot[t][4 * a + 2 * b + 1], 0.00048828125f, tot[t][4 * a + 2 * b]);
+  if (kparts == 1u) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const u32 token = (tg * NT + t) * kTokensPerTile + 4u * a + 2u * g + b;
+          if (row_ok && token < m) c[static_cast<size_t>(token) * n + row] = val[t][2 * a + b];
+        }
     return;
   }
   // The parts cross workgroups (and XCDs): 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side
@@ -209,55 +215,72 @@ __device__ __forceinline__ void finish_tile(const f32x16& tot, float* __restrict
   const u32 strips = groups * waves;
   const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       ws + kCounterBytes, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
-  auto slot_of = [&](u32 pt) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
-  __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[0]), __float_as_uint(val[1]), __float_as_uint(val[2]), __float_as_uint(val[3])},
-                                         part_rsrc, slot_of(part), 0, 16);
-  const bool upper = tile * kTokensPerTile + 8u < m;      // tokens 8..15 of the tile exist (val[4..7])
-  if (upper)
-    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[4]), __float_as_uint(val[5]), __float_as_uint(val[6]), __float_as_uint(val[7])},
-                                           part_rsrc, slot_of(part) + 16, 0, 16);
+  auto slot_of = [&](u32 pt, u32 tile) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
+  bool lower[NT], upper[NT];      // tokens 0..7 / 8..15 of the tile exist (val[0..3] / val[4..7])
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const u32 tile = tg * NT + t;
+    lower[t] = tile * kTokensPerTile < m;
+    upper[t] = tile * kTokensPerTile + 8u < m;
+    if (lower[t])
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[t][0]), __float_as_uint(val[t][1]), __float_as_uint(val[t][2]), __float_as_uint(val[t][3])},
+                                             part_rsrc, slot_of(part, tile), 0, 16);
+    if (upper[t])
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[t][4]), __float_as_uint(val[t][5]), __float_as_uint(val[t][6]), __float_as_uint(val[t][7])},
+                                             part_rsrc, slot_of(part, tile) + 16, 0, 16);
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
   asm volatile("s_barrier" ::: "memory");
   if (threadIdx.x == 0u) {
-    const u32 old = __hip_atomic_fetch_add(counters + group * tiles + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const u32 old = __hip_atomic_fetch_add(counters + group * tgroups + tg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(lds_flag), "v"(old) : "memory");
   }
   asm volatile("s_barrier" ::: "memory");
   u32 old;
   asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(lds_flag) : "memory");
   if (old == kparts - 1u && threadIdx.x == 0u)      // ready for the next product on this stream
-    __hip_atomic_store(counters + group * tiles + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(counters + group * tgroups + tg, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (old != kparts - 1u || !row_ok) return;
-  float r[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-  // all parts in flight at once when they are at most sixteen (a round trip to memory each time otherwise), added in
-  // part order; no more loads than there are parts to the next power of two
+  float r[NT][8];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[t][e] = 0.0f;
+  // all parts in flight at once when they are few (a round trip to memory each time otherwise), added in part order;
+  // no more loads than there are parts to the next power of two
   auto add_parts = [&](auto width) {
     constexpr u32 W = decltype(width)::value;
     for (u32 p0 = 0; p0 < kparts; p0 += W) {
-      u32x4 lo[W], hi[W];
+      u32x4 lo[NT][W], hi[NT][W];
 #pragma unroll
-      for (u32 pp = 0; pp < W; ++pp) {
-        const u32 pt = min(p0 + pp, kparts - 1u);
-        lo[pp] = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt), 0, 16);
-        hi[pp] = upper ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
-      }
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (u32 pp = 0; pp < W; ++pp)
-        if (p0 + pp < kparts) {
-          r[0] += __uint_as_float(lo[pp].x); r[1] += __uint_as_float(lo[pp].y); r[2] += __uint_as_float(lo[pp].z); r[3] += __uint_as_float(lo[pp].w);
-          r[4] += __uint_as_float(hi[pp].x); r[5] += __uint_as_float(hi[pp].y); r[6] += __uint_as_float(hi[pp].z); r[7] += __uint_as_float(hi[pp].w);
+        for (u32 pp = 0; pp < W; ++pp) {
+          const u32 pt = min(p0 + pp, kparts - 1u);
+          lo[t][pp] = lower[t] ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt, tg * NT + t), 0, 16) : u32x4{0u, 0u, 0u, 0u};
+          hi[t][pp] = upper[t] ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt, tg * NT + t) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
         }
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (u32 pp = 0; pp < W; ++pp)
+          if (p0 + pp < kparts) {
+            r[t][0] += __uint_as_float(lo[t][pp].x); r[t][1] += __uint_as_float(lo[t][pp].y); r[t][2] += __uint_as_float(lo[t][pp].z); r[t][3] += __uint_as_float(lo[t][pp].w);
+            r[t][4] += __uint_as_float(hi[t][pp].x); r[t][5] += __uint_as_float(hi[t][pp].y); r[t][6] += __uint_as_float(hi[t][pp].z); r[t][7] += __uint_as_float(hi[t][pp].w);
+          }
     }
   };
   if (kparts <= 2u) add_parts(std::integral_constant<u32, 2>{});
   else if (kparts <= 4u) add_parts(std::integral_constant<u32, 4>{});
-  else if (kparts <= 8u) add_parts(std::integral_constant<u32, 8>{});
+  else if (kparts <= 8u || NT > 1) add_parts(std::integral_constant<u32, 8>{});
   else add_parts(std::integral_constant<u32, 16>{});
 #pragma unroll
-  for (int t = 0; t < 8; ++t) {
-    const u32 token = tile * kTokensPerTile + 4u * (t >> 1) + 2u * g + (t & 1);
-    if (token < m) c[static_cast<size_t>(token) * n + row] = r[t];
-  }
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const u32 token = (tg * NT + t) * kTokensPerTile + 4u * (e >> 1) + 2u * g + (e & 1);
+      if (token < m) c[static_cast<size_t>(token) * n + row] = r[t][e];
+    }
 }
 
 // What every kernel of this file takes: the operands, the workspace (counters, then partial sums), the shape and
@@ -270,13 +293,13 @@ struct Geometry {
         groups(static_cast<u32>(geom >> 32) & 0xFFFFu), tiles(static_cast<u32>(geom >> 48)) {}
 };
 
-// Main kernel.  Workgroup id -> (unit, token tile) with the token tiles of a unit 8 ids apart (same XCD, so the
-// weights they share meet in that XCD's L2); unit -> (group of 8 strips, part of K).  With one part the result
-// is stored; otherwise every part stores its partial result in `partial`, and the workgroup that arrives last
-// at the (group, tile) counter adds the parts in part order - the sum does not depend on who is last - and
-// puts the counter back to zero (the counters start at zero when the workspace is allocated).
-//   dynamic LDS = kLdsBytes
-template <int FMT, int CHUNKS>     // CHUNKS: chunks of A a thread converts per super-block, 512 / threads
+// Main kernel.  Workgroup id -> (unit, tile group) with the tile groups of a unit 8 ids apart (same XCD, so the
+// weights they share meet in that XCD's L2); unit -> (group of 8 strips, part of K).  A workgroup takes NT token
+// tiles (a tile group): the weight operands of a product are built once and meet NT tiles' tokens, which is what
+// pays when the tokens are many - building them is most of a super-block's instructions.  (finish_tiles: what
+// happens with the results.)
+//   dynamic LDS = lds_bytes(waves, tile bytes, NT)
+template <int FMT, int CHUNKS, int NT>     // CHUNKS: chunks of A a thread converts per super-block and tile, 512 / threads
 __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, uint8_t* __restrict__ ws,
                                          u32 m, u32 n, u32 nsb, uint64_t geom, u32 lds_base) {
   const Geometry cut(geom);
@@ -284,7 +307,8 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   const u32 lane = threadIdx.x & 63u;
   const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6)));
   const u32 id = blockIdx.x;
-  const u32 unit = (id / (8u * tiles)) * 8u + (id & 7u), tile = (id >> 3) % tiles;
+  const u32 tgroups = (tiles + NT - 1u) / NT;
+  const u32 unit = (id / (8u * tgroups)) * 8u + (id & 7u), tg = (id >> 3) % tgroups;
   if (unit >= groups * kparts) return;
   const u32 group = unit / kparts, part = unit - group * kparts;
   const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
@@ -304,19 +328,21 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     const u32 r = p / T::PIECES, cc = p - T::PIECES * r;
     woff[t] = static_cast<size_t>(min(strip * 32u + r, n - 1u)) * row_bytes + 16u * cc;
   }
-  const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kXpStageBytes + wave * (2u * kWStageBytes);
-  const u32 lds_flag = lds_base + 2u * kXpStageBytes + 2u * waves * kWStageBytes;
+  constexpr u32 kStage = NT * kXpStageBytes;      // the token operands of one super-block: NT tiles one behind the other
+  const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kStage + wave * (2u * kWStageBytes);
+  const u32 lds_flag = lds_base + 2u * kStage + 2u * waves * kWStageBytes;
   // the chunks of A this thread converts per super-block: 512 chunks of 8 elements (16 tokens x 32)
   constexpr u32 nthreads = 512u / CHUNKS;
-  const float* asrc[CHUNKS];
-  u32 ctoken[CHUNKS], cpos[CHUNKS];
-  bool live[CHUNKS];
+  constexpr int NC = CHUNKS * NT;      // chunk i: tile i / CHUNKS of the group
+  const float* asrc[NC];
+  u32 ctoken[NC], cpos[NC];
+  bool live[NC];
 #pragma unroll
-  for (int i = 0; i < CHUNKS; ++i) {
-    const u32 idx = threadIdx.x + i * nthreads;
+  for (int i = 0; i < NC; ++i) {
+    const u32 idx = threadIdx.x + (i % CHUNKS) * nthreads;
     ctoken[i] = (idx >> 5) & 15u;
     cpos[i] = idx & 31u;
-    const u32 token = tile * kTokensPerTile + ctoken[i];
+    const u32 token = (tg * NT + i / CHUNKS) * kTokensPerTile + ctoken[i];
     asrc[i] = a + static_cast<size_t>(min(token, m - 1u)) * (static_cast<size_t>(nsb) * 256u) + 8u * cpos[i];
     live[i] = token < m;
   }
@@ -329,10 +355,10 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     for (int t = 0; t < DMA - 1; ++t) dma16(wsrc + woff[t], wl + 1024u * t);
     if (lane < 32u) dma16(wsrc + woff[DMA - 1], wl + 1024u * (DMA - 1));
   };
-  u32x4 an[CHUNKS][2];                 // A of a super-block on its way to conversion
+  u32x4 an[NC][2];                     // A of a super-block on its way to conversion
   auto load_a = [&](u32 s) {
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
+    for (int i = 0; i < NC; ++i) {
       const float* src = asrc[i] + static_cast<size_t>(sb0 + s) * 256u;
       asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
                    : "=&v"(an[i][0]), "=&v"(an[i][1]) : "v"(src) : "memory");
@@ -340,17 +366,19 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   };
   auto convert = [&](u32 s) {          // the loads of A issued last have landed when DMA loads (of W) are left
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA) : "memory");
+    for (int i = 0; i < NC; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA) : "memory");
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i)
+    for (int i = 0; i < NC; ++i)
       convert_chunk(live[i] ? __builtin_bit_cast(f32x4, an[i][0]) : zero4, live[i] ? __builtin_bit_cast(f32x4, an[i][1]) : zero4,
-                    ctoken[i], cpos[i], lds_xp + (s & 1u) * kXpStageBytes);
+                    ctoken[i], cpos[i], lds_xp + (s & 1u) * kStage + (i / CHUNKS) * kXpStageBytes);
   };
 
-  f32x16 tot;
+  f32x16 tot[NT];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) tot[v] = 0.0f;
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) tot[t][v] = 0.0f;
   u32 xq[16];                                    // where this lane finds its token operands of product q (stage 0)
 #pragma unroll
   for (u32 q = 0; q < 16; ++q) xq[q] = lds_xp + ((lane ^ (2u * q)) << 4);
@@ -364,30 +392,34 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   }
   for (u32 s = 0; s < ns; ++s) {
     // weight tile s has landed (the loads of super-block s+1 may be in flight); the token operands of s are written
-    if (s + 1u < ns) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * CHUNKS + DMA) : "memory");
+    if (s + 1u < ns) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NC + DMA) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     asm volatile("s_barrier" ::: "memory");
     const u32 slot = s & 1u;
     const u32 wt = lds_w + slot * kWStageBytes + col * T::SB, wl = wt + g * 64u;
-    const u32 xl = lds_xp + slot * kXpStageBytes + lane * 16u;
-    const u32 sl = lds_xp + slot * kXpStageBytes + kXpMainBytes + lane * 8u;
-    const u32 fl = lds_xp + slot * kXpStageBytes + kXpMainBytes + kXpSumBytes + g * 8u;
+    const u32 sl = lds_xp + slot * kStage + kXpMainBytes + lane * 8u;
+    const u32 fl = lds_xp + slot * kStage + kXpMainBytes + kXpSumBytes + g * 8u;
     u32x4 hdr, d0, d1, d2, d3;
-    u32x2 sx, f01, f23, f45, f67;
+    u32x2 sx[NT], f01[NT], f23[NT], f45[NT], f67[NT];
     asm volatile("ds_read_b128 %0, %1" : "=&v"(hdr) : "v"(wt) : "memory");
     lds_read128<16>(d0, wl);
     lds_read128<32>(d1, wl);
     lds_read128<48>(d2, wl);
     lds_read128<64>(d3, wl);
-    lds_read64<0>(sx, sl);
-    lds_read64<0>(f01, fl);          // 2^(E+14) of the tokens 4a + 2g + {0, 1}, a = 0..3
-    lds_read64<16>(f23, fl);
-    lds_read64<32>(f45, fl);
-    lds_read64<48>(f67, fl);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      lds_read64<0>(sx[t], sl + t * kXpStageBytes);
+      lds_read64<0>(f01[t], fl + t * kXpStageBytes);          // 2^(E+14) of the tokens 4a + 2g + {0, 1}, a = 0..3
+      lds_read64<16>(f23[t], fl + t * kXpStageBytes);
+      lds_read64<32>(f45[t], fl + t * kXpStageBytes);
+      lds_read64<48>(f67[t], fl + t * kXpStageBytes);
+    }
     [[maybe_unused]] u32x4 qh = {0u, 0u, 0u, 0u};      // Q5_K: this lane group's 16 bytes of fifth bits (values 128 g .. 128 g + 127)
     if constexpr (FMT == FMT_Q5K) lds_read128<144>(qh, wt + g * 16u);
-    lds_wait5(hdr, d0, d1, d2, d3, sx);
-    asm volatile("" : "+v"(f01), "+v"(f23), "+v"(f45), "+v"(f67), "+v"(qh));
+    lds_wait5(hdr, d0, d1, d2, d3, sx[0]);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) asm volatile("" : "+v"(sx[t]), "+v"(f01[t]), "+v"(f23[t]), "+v"(f45[t]), "+v"(f67[t]));
+    asm volatile("" : "+v"(qh));
     if (s + 1u < ns) convert(s + 1u);        // into the stage that was read two super-blocks ago
     if (s + 2u < ns) {          // the weight tile is in registers: its LDS space takes the tile after the next
       load_a(s + 2u);
@@ -419,19 +451,25 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
                       static_cast<_Float16>(static_cast<unsigned short>((m4 >> 16) & 0xFFu)),
                       static_cast<_Float16>(static_cast<unsigned short>(m4 >> 24))};
     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    const f32x16 macc = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx), mb, zero, 0, 0, 0);
-    f32x16 acc = zero;
+    f32x16 macc[NT], acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      macc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx[t]), mb, zero, 0, 0, 0);
+      acc[t] = zero;
+    }
 #pragma unroll
     for (int uu = 0; uu < 8; uu += 2) {          // two dword pairs = four products per round of operand reads
-      u32x4 a0, a1, a2, a3;
-      const u32 xs = slot * kXpStageBytes;       // product q reads slot lane ^ 2q of its page (xq[q], set up once)
-      switch (uu) {
-        case 0: lds_read128<0 * 1024>(a0, xq[0] + xs); lds_read128<1 * 1024>(a1, xq[1] + xs); lds_read128<2 * 1024>(a2, xq[2] + xs); lds_read128<3 * 1024>(a3, xq[3] + xs); break;
-        case 2: lds_read128<4 * 1024>(a0, xq[4] + xs); lds_read128<5 * 1024>(a1, xq[5] + xs); lds_read128<6 * 1024>(a2, xq[6] + xs); lds_read128<7 * 1024>(a3, xq[7] + xs); break;
-        case 4: lds_read128<8 * 1024>(a0, xq[8] + xs); lds_read128<9 * 1024>(a1, xq[9] + xs); lds_read128<10 * 1024>(a2, xq[10] + xs); lds_read128<11 * 1024>(a3, xq[11] + xs); break;
-        default: lds_read128<12 * 1024>(a0, xq[12] + xs); lds_read128<13 * 1024>(a1, xq[13] + xs); lds_read128<14 * 1024>(a2, xq[14] + xs); lds_read128<15 * 1024>(a3, xq[15] + xs); break;
+      u32x4 ax[NT][4];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32 xs = slot * kStage + t * kXpStageBytes;       // product q reads slot lane ^ 2q of its page (xq[q], set up once)
+        switch (uu) {
+          case 0: lds_read128<0 * 1024>(ax[t][0], xq[0] + xs); lds_read128<1 * 1024>(ax[t][1], xq[1] + xs); lds_read128<2 * 1024>(ax[t][2], xq[2] + xs); lds_read128<3 * 1024>(ax[t][3], xq[3] + xs); break;
+          case 2: lds_read128<4 * 1024>(ax[t][0], xq[4] + xs); lds_read128<5 * 1024>(ax[t][1], xq[5] + xs); lds_read128<6 * 1024>(ax[t][2], xq[6] + xs); lds_read128<7 * 1024>(ax[t][3], xq[7] + xs); break;
+          case 4: lds_read128<8 * 1024>(ax[t][0], xq[8] + xs); lds_read128<9 * 1024>(ax[t][1], xq[9] + xs); lds_read128<10 * 1024>(ax[t][2], xq[10] + xs); lds_read128<11 * 1024>(ax[t][3], xq[11] + xs); break;
+          default: lds_read128<12 * 1024>(ax[t][0], xq[12] + xs); lds_read128<13 * 1024>(ax[t][1], xq[13] + xs); lds_read128<14 * 1024>(ax[t][2], xq[14] + xs); lds_read128<15 * 1024>(ax[t][3], xq[15] + xs); break;
+        }
       }
-      const u32x4* aq[4] = {&a0, &a1, &a2, &a3};
       u32 bl[2][4], bh[2][4];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -463,26 +501,34 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
         bh[i][2] = __builtin_bit_cast(u32, pk_mul_h2((t1 & 0x00F000F0u) | e[1][0], sh2));
         bh[i][3] = __builtin_bit_cast(u32, pk_mul_h2((t1s & 0x00F000F0u) | e[1][1], sh2));
       }
-      lds_wait4(a0, a1, a2, a3);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) lds_wait4(ax[t][0], ax[t][1], ax[t][2], ax[t][3]);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const u32x4 blv = {bl[i][0], bl[i][1], bl[i][2], bl[i][3]}, bhv = {bh[i][0], bh[i][1], bh[i][2], bh[i][3]};
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[2 * i]), __builtin_bit_cast(h16x8, blv), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, *aq[2 * i + 1]), __builtin_bit_cast(h16x8, bhv), acc, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, ax[t][2 * i]), __builtin_bit_cast(h16x8, blv), acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, ax[t][2 * i + 1]), __builtin_bit_cast(h16x8, bhv), acc[t], 0, 0, 0);
       }
     }
     const float nm = dmin * -0.001953125f;       // -dmin * 2^-9: the sums carry 2^-5, the products 2^-14
-    const float fac[8] = {__uint_as_float(f01.x), __uint_as_float(f01.y), __uint_as_float(f23.x), __uint_as_float(f23.y),
-                          __uint_as_float(f45.x), __uint_as_float(f45.y), __uint_as_float(f67.x), __uint_as_float(f67.y)};
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const float fd = fac[t] * d, fm = fac[t] * nm;
-      tot[2 * t] = fmaf(fm, macc[2 * t], fmaf(fd, acc[2 * t], tot[2 * t]));
-      tot[2 * t + 1] = fmaf(fm, macc[2 * t + 1], fmaf(fd, acc[2 * t + 1], tot[2 * t + 1]));
+    for (int t = 0; t < NT; ++t) {
+      const float fac[8] = {__uint_as_float(f01[t].x), __uint_as_float(f01[t].y), __uint_as_float(f23[t].x), __uint_as_float(f23[t].y),
+                            __uint_as_float(f45[t].x), __uint_as_float(f45[t].y), __uint_as_float(f67[t].x), __uint_as_float(f67[t].y)};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float fd = fac[e] * d, fm = fac[e] * nm;
+        tot[t][2 * e] = fmaf(fm, macc[t][2 * e], fmaf(fd, acc[t][2 * e], tot[t][2 * e]));
+        tot[t][2 * e + 1] = fmaf(fm, macc[t][2 * e + 1], fmaf(fd, acc[t][2 * e + 1], tot[t][2 * e + 1]));
+      }
     }
   }
 
-  finish_tile(tot, c, ws, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
+  finish_tiles<NT>(tot, c, ws, m, n, kparts, groups, tiles, tgroups, waves, group, part, tg, strip, col, g, lane, lds_flag);
 }
 
 
@@ -715,7 +761,8 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
     step(s, true_type{}, false_type{});
     step(s + 1u, false_type{}, false_type{});
   }
-  finish_tile(tot, c, ws, m, n, kparts, groups, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
+  const f32x16 tots[1] = {tot};
+  finish_tiles<1>(tots, c, ws, m, n, kparts, groups, tiles, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
 }
 
 }  // namespace gemm_f16

@@ -77,6 +77,7 @@ struct DeviceKernels {
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
   hipFunction_t gemm_f16[NFMT][2] = {};   // [format][4 or 8 strips per workgroup]
+  hipFunction_t gemm_f16_t2[2] = {};      // Q4_K, Q5_K: 8 strips and two token tiles per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
@@ -92,6 +93,7 @@ std::atomic<int> g_tune_group_off{0};
 std::atomic<int> g_tune_group_pool_off{0};
 std::atomic<int> g_tune_group_pool_waves{0};  // 1: grouped launches cut every entry's rows evenly (no run-time pools)
 std::atomic<int> g_tune_gemm_mfma_off{0};   // 1: the Q4_K GEMM never takes the matrix-core form
+std::atomic<int> g_tune_gemm_tiles{0};      // token tiles per workgroup of the matrix-core GEMM: 0 by the rule, 1, 2
 std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 std::atomic<int> g_tune_attention_min_steps{0};
 std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped launch may look ahead over (0: 16)
@@ -157,6 +159,8 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.gemm_f16[0][1], "q4k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[1][0], "q5k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[1][1], "q5k_gemm_f16_w8")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16_t2[0], "q4k_gemm_f16_w8t2")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16_t2[1], "q5k_gemm_f16_w8t2")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][0], "q6k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][1], "q6k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
@@ -379,18 +383,41 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   const uint32_t kGemmQ6TileBytes = 32u * 240u;
   // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
   const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
-  const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
-                                : 2u * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
   const uint32_t groups = (n + 32u * waves - 1u) / (32u * waves);
-  // cut K so that the workgroups are about as many as the CUs
-  const uint64_t units = uint64_t(groups) * tiles;
-  uint32_t kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d->cu_count) + units / 2u) / units);
-  kparts = std::min(std::max(kparts, 1u), nsb);
-  const uint32_t ksb = (nsb + kparts - 1u) / kparts;
-  kparts = (nsb + ksb - 1u) / ksb;
+  // How the product is cut: nt token tiles of 16 per workgroup (tgroups tile groups), K in kparts parts of ksb
+  // super-blocks, so that the workgroups are about as many as the CUs.
+  struct Cut { uint32_t nt, tgroups, kparts, ksb; double us; };
+  auto cut_for = [&](uint32_t nt) {
+    Cut c{nt, (tiles + nt - 1u) / nt, 1u, nsb, 0.0};
+    const uint64_t units = uint64_t(groups) * c.tgroups;
+    c.kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d->cu_count) + units / 2u) / units);
+    c.kparts = std::min(std::max(c.kparts, 1u), nsb);
+    c.ksb = (nsb + c.kparts - 1u) / c.kparts;
+    c.kparts = (nsb + c.ksb - 1u) / c.ksb;
+    // Time in microseconds, fitted to measurements on MI355X (Q4_K, 4096 x 4096 .. 14336 x 4096, 32 .. 512 tokens): 6 to
+    // the first super-block and for the stores; a super-block takes a workgroup 2.0 with one tile and 3.2 with two
+    // (the weight operands are built once for both); with K in parts 4 more for the sum over the parts, 3 for every
+    // further round of eight (two tiles) or sixteen parts in flight, and 4 for the second tile's share of it.
+    const uint64_t rounds = (units * c.kparts + uint64_t(d->cu_count) - 1u) / uint64_t(d->cu_count);
+    const uint32_t in_flight = nt == 2u ? 8u : 16u;
+    c.us = 6.0 + double(rounds) * c.ksb * (nt == 2u ? 3.2 : 2.0) +
+           (c.kparts > 1u ? 4.0 + 3.0 * ((c.kparts + in_flight - 1u) / in_flight - 1u) + (nt == 2u ? 4.0 : 0.0) : 0.0);
+    return c;
+  };
+  // Two tiles per workgroup: Q4_K and Q5_K (the Q6_K kernel has no registers left for it), where the estimate says so
+  // (14336 x 4096: M = 48 41 -> 32 us, M = 128 65 -> 52 us, M = 512 234 -> 204 us; where K has to be cut finer instead
+  // it is slower, 4096 x 4096, M = 32: 14.5 -> 22.4 us)
+  Cut cut = cut_for(1u);
+  if (waves == 8u && f != Q6K && tiles >= 2u && g_tune_gemm_tiles != 1) {
+    const Cut two = cut_for(2u);
+    if (g_tune_gemm_tiles == 2 || two.us < cut.us) cut = two;
+  }
+  const uint32_t nt = cut.nt, tgroups = cut.tgroups, kparts = cut.kparts, ksb = cut.ksb;
+  const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
+                                : 2u * nt * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
   auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
   // with several parts of K: one arrival counter per (group of strips, token tile)
-  const size_t cnt_bytes = kparts > 1u ? size_t(groups) * tiles * 4u : 0u;
+  const size_t cnt_bytes = kparts > 1u ? size_t(groups) * tgroups * 4u : 0u;
   // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
   const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * groups * waves * 2048u) : 0u;
   // the counters sit at the front of a region that only grows, so a larger product finds zeros there too (the
@@ -405,11 +432,12 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
     if (e != hipSuccess) return e;
   }
   const uint64_t padded = (uint64_t(groups) * kparts + 7u) / 8u * 8u;
-  if (ksb > 0xFFFFu || groups > 0xFFFFu || tiles > 0xFFFFu || padded * tiles > 0x7FFFFFFFu) return hipErrorInvalidValue;
+  if (ksb > 0xFFFFu || groups > 0xFFFFu || tiles > 0xFFFFu || padded * tgroups > 0x7FFFFFFFu) return hipErrorInvalidValue;
   uint32_t nsb_arg = nsb;
   uint64_t geom = uint64_t(ksb) | uint64_t(kparts) << 16 | uint64_t(groups) << 32 | uint64_t(tiles) << 48;
   void* margs[] = {&a, &w, &c, &cnt, &m, &n, &nsb_arg, &geom};
-  return hipModuleLaunchKernel(d->gemm_f16[f][waves == 8u], uint32_t(padded * tiles), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
+  hipFunction_t fn = nt == 2u ? d->gemm_f16_t2[f] : d->gemm_f16[f][waves == 8u];
+  return hipModuleLaunchKernel(fn, uint32_t(padded * tgroups), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
 // does the matrix-core form take this product?  (weights 16-byte aligned; Q6_K, whose blocks are 210 bytes, 2-byte aligned)
@@ -439,7 +467,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
   if (!is_gemv && q4k_gemm_f16_ok(a, w, c, m, n, k, f) &&
-      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || !gemm_few_tokens_by_engine(f, m, n, k)))
+      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0 || !gemm_few_tokens_by_engine(f, m, n, k)))
     return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
@@ -1483,6 +1511,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "chain_spin_limit")) { g_tune_chain_spin_limit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_off")) { g_tune_group_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_mfma_off")) { g_tune_gemm_mfma_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_tiles")) { g_tune_gemm_tiles = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_k_parts")) { g_tune_gemm_ksplit = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_window")) { g_tune_group_window = value; return TRN_SUCCESS; }
