@@ -373,6 +373,48 @@ ScratchMap g_gemm_ws;
 constexpr uint32_t kGemmXpStageBytes = 16 * 1024 + 512 + 64;
 constexpr size_t kGemmCounterBytes = size_t(1) << 16;   // arrival counters at the front of the GEMM's scratch buffer
 
+// How a product on the matrix cores is cut: `waves` strips of 32 rows and nt token tiles of 16 per workgroup (groups of
+// strips, tgroups of tiles), K in kparts parts of ksb super-blocks, so that the workgroups are about as many as the CUs.
+struct GemmCut { uint32_t waves, nt, groups, tgroups, kparts, ksb; double us; };
+
+// The cut with the least estimated time among: 8 strips and one tile, 8 strips and two tiles (Q4_K and Q5_K: the weight
+// operands are built once for both; the Q6_K kernel has no registers left for it), 4 strips and one tile.  Times in
+// microseconds fitted to measurements on MI355X (Q4_K, 1024 x 4096 .. 14336 x 4096 and 4096 x 14336, 4 .. 512 tokens; they
+// hold within about 15 %): 5 to the first super-block and for the stores (3.5 with 4 strips); a super-block takes a
+// workgroup 2.0 (8 strips), 3.2 (8 strips, two tiles) or 1.5 (4 strips); with K in parts 2.5 for publishing a part, plus the time in
+// which the workgroup that arrives last reads every part of its rows through one CU, at about 40 GB/s - with 16 parts
+// of 8 strips that read alone took 6.5 us of 15 (4096 x 4096, M = 16: 15.0 us with 8 strips, 10.3 us with 4).
+// Examples (us, 8 strips and one tile -> chosen): 4096 x 4096 M = 16 15.0 -> 10.3; 1024 x 4096 M = 64 14.6 -> 9.8;
+// 14336 x 4096 M = 48 41 -> 32, M = 128 65 -> 53, M = 512 234 -> 201; 4096 x 4096 M = 32 with two tiles would be 22.4
+// against 13.
+GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t k) {
+  const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
+  auto cut_for = [&](uint32_t waves, uint32_t nt) {
+    GemmCut c{waves, nt, (n + 32u * waves - 1u) / (32u * waves), (tiles + nt - 1u) / nt, 1u, nsb, 0.0};
+    const uint64_t units = uint64_t(c.groups) * c.tgroups;
+    c.kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d.cu_count) + units / 2u) / units);
+    c.kparts = std::min(std::max(c.kparts, 1u), nsb);
+    c.ksb = (nsb + c.kparts - 1u) / c.kparts;
+    c.kparts = (nsb + c.ksb - 1u) / c.ksb;
+    const uint64_t rounds = (units * c.kparts + uint64_t(d.cu_count) - 1u) / uint64_t(d.cu_count);
+    const double step = waves == 4u ? 1.5 : nt == 2u ? 3.2 : 2.0;
+    const double last_kb = double(c.kparts) * waves * nt * (m > 8u ? 2.0 : 1.0);
+    c.us = (waves == 4u ? 3.5 : 5.0) + double(rounds) * c.ksb * step + (c.kparts > 1u ? 2.5 + last_kb / 40.0 : 0.0);
+    return c;
+  };
+  const int tw = g_tune_gemm_waves, tt = g_tune_gemm_tiles;
+  GemmCut best = cut_for(tw == 4 ? 4u : 8u, 1u);
+  if (tw == 0 && tt != 2) {
+    const GemmCut four = cut_for(4u, 1u);
+    if (four.us < best.us) best = four;
+  }
+  if (tw != 4 && f != Q6K && tiles >= 2u && tt != 1) {
+    const GemmCut two = cut_for(8u, 2u);
+    if (tt == 2 || two.us < best.us) best = two;
+  }
+  return best;
+}
+
 // ext_base != 0: the caller brings the scratch buffer (ext_cap bytes, counters at its front already zero); nothing is
 // allocated and a product that needs more is refused.
 hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
@@ -381,38 +423,8 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   const uint32_t kGemmWTileBytes = 32u * kSbBytes[f];
   // Q6_K: one weight tile per wave, rows 240 bytes apart (q6k_lds_bytes of the kernel's header)
   const uint32_t kGemmQ6TileBytes = 32u * 240u;
-  // strips of 32 rows per workgroup: 8 share the token operands best (4 measured no better on any shape tried)
-  const uint32_t waves = g_tune_gemm_waves == 4 ? 4u : 8u;
-  const uint32_t groups = (n + 32u * waves - 1u) / (32u * waves);
-  // How the product is cut: nt token tiles of 16 per workgroup (tgroups tile groups), K in kparts parts of ksb
-  // super-blocks, so that the workgroups are about as many as the CUs.
-  struct Cut { uint32_t nt, tgroups, kparts, ksb; double us; };
-  auto cut_for = [&](uint32_t nt) {
-    Cut c{nt, (tiles + nt - 1u) / nt, 1u, nsb, 0.0};
-    const uint64_t units = uint64_t(groups) * c.tgroups;
-    c.kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d->cu_count) + units / 2u) / units);
-    c.kparts = std::min(std::max(c.kparts, 1u), nsb);
-    c.ksb = (nsb + c.kparts - 1u) / c.kparts;
-    c.kparts = (nsb + c.ksb - 1u) / c.ksb;
-    // Time in microseconds, fitted to measurements on MI355X (Q4_K, 4096 x 4096 .. 14336 x 4096, 32 .. 512 tokens): 6 to
-    // the first super-block and for the stores; a super-block takes a workgroup 2.0 with one tile and 3.2 with two
-    // (the weight operands are built once for both); with K in parts 4 more for the sum over the parts, 3 for every
-    // further round of eight (two tiles) or sixteen parts in flight, and 4 for the second tile's share of it.
-    const uint64_t rounds = (units * c.kparts + uint64_t(d->cu_count) - 1u) / uint64_t(d->cu_count);
-    const uint32_t in_flight = nt == 2u ? 8u : 16u;
-    c.us = 6.0 + double(rounds) * c.ksb * (nt == 2u ? 3.2 : 2.0) +
-           (c.kparts > 1u ? 4.0 + 3.0 * ((c.kparts + in_flight - 1u) / in_flight - 1u) + (nt == 2u ? 4.0 : 0.0) : 0.0);
-    return c;
-  };
-  // Two tiles per workgroup: Q4_K and Q5_K (the Q6_K kernel has no registers left for it), where the estimate says so
-  // (14336 x 4096: M = 48 41 -> 32 us, M = 128 65 -> 52 us, M = 512 234 -> 204 us; where K has to be cut finer instead
-  // it is slower, 4096 x 4096, M = 32: 14.5 -> 22.4 us)
-  Cut cut = cut_for(1u);
-  if (waves == 8u && f != Q6K && tiles >= 2u && g_tune_gemm_tiles != 1) {
-    const Cut two = cut_for(2u);
-    if (g_tune_gemm_tiles == 2 || two.us < cut.us) cut = two;
-  }
-  const uint32_t nt = cut.nt, tgroups = cut.tgroups, kparts = cut.kparts, ksb = cut.ksb;
+  const GemmCut cut = gemm_cut(*d, f, m, n, k);
+  const uint32_t waves = cut.waves, nt = cut.nt, groups = cut.groups, tgroups = cut.tgroups, kparts = cut.kparts, ksb = cut.ksb;
   const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
                                 : 2u * nt * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
   auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
@@ -449,13 +461,15 @@ bool q4k_gemm_f16_ok(uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
 
 // A few tokens against a small matrix are faster through the GEMV engine, one pass per token with the weights of the
 // second and later passes coming from the caches, than through the matrix-core kernel with its start-up and its sum
-// over the parts of K.  Times in microseconds fitted to measurements on MI355X (MB = weight bytes / 1e6):
-//   engine: 3.9 + MB / 5.7 for the first token, MB / 5.8 + 0.15 for each further one (one slab of columns only; with
-//   k > 4096 a further pass costs as much as the first); matrix cores: 12 + MB / 9.4 for up to 16 tokens.
-bool gemm_few_tokens_by_engine(Fmt f, uint32_t m, uint32_t n, uint32_t k) {
+// over the parts of K.  The engine's time in microseconds, fitted to measurements on MI355X (MB = weight bytes / 1e6):
+// 3.9 + MB / 5.7 for the first token, MB / 5.8 + 0.15 for each further one (one slab of columns only; with k > 4096 a
+// further pass costs as much as the first); the matrix cores' for up to 16 tokens, where the weights' bytes still
+// count: 7.2 + MB / 4 with 4 strips per workgroup, 12 + MB / 9.4 with 8.
+bool gemm_few_tokens_by_engine(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t k) {
   if (m > 8u || k > 4096u) return false;
   const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
-  return 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15) < 12.0 + mb / 9.4;
+  const double matrix_cores = gemm_cut(d, f, m, n, k).waves == 4u ? 7.2 + mb / 4.0 : 12.0 + mb / 9.4;
+  return 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15) < matrix_cores;
 }
 
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
@@ -467,7 +481,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
   if (!is_gemv && q4k_gemm_f16_ok(a, w, c, m, n, k, f) &&
-      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0 || !gemm_few_tokens_by_engine(f, m, n, k)))
+      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0 || !gemm_few_tokens_by_engine(*d, f, m, n, k)))
     return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
@@ -1395,11 +1409,12 @@ trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c
   if (n == 0 || m == 0) return TRN_SUCCESS;
   if ((a == 0 && k != 0) || c == 0 || (b == 0 && k != 0)) return TRN_ERROR_INVALID_VALUE;
   hipStream_t stream = static_cast<hipStream_t>(s);
-  // the same choice of kernel as trn_q4k_gemm, so the same bits: the GEMV engine needs no scratch at all
-  if (!q4k_gemm_f16_ok(a, b, c, m, n, k) || (g_tune_gemm_ksplit == 0 && g_tune_gemm_waves == 0 && gemm_few_tokens_by_engine(Q4K, m, n, k)))
-    return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));
   DeviceKernels* d = nullptr;
   TRN_TRY(device_kernels(&d));
+  // the same choice of kernel as trn_q4k_gemm, so the same bits: the GEMV engine needs no scratch at all
+  if (!q4k_gemm_f16_ok(a, b, c, m, n, k) ||
+      (g_tune_gemm_ksplit == 0 && g_tune_gemm_waves == 0 && g_tune_gemm_tiles == 0 && gemm_few_tokens_by_engine(*d, Q4K, m, n, k)))
+    return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));
   int dev = 0;
   TRN_TRY(hipGetDevice(&dev));
   size_t cap = 0;
