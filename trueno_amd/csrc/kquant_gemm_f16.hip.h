@@ -347,7 +347,11 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     live[i] = token < m;
   }
 
-  // Loads are counted by hand (s_waitcnt vmcnt): per super-block a wave issues 2*CHUNKS loads of A, then DMA of W.
+  // Loads are counted by hand (s_waitcnt vmcnt): per super-block a wave issues 2*NC loads of A, then DMA of W.  (With
+  // ordinary loads of A the compiler waits for vmcnt(0) wherever DMA is also in flight, which takes the copies of W out
+  // of the background.  The price of asm: between such a load and the wait that names its registers the compiler must
+  // have no reason to copy them - one definition per loop, no second set of registers joined to the first; a variant
+  // that requested two super-blocks up front broke exactly there, and the parity tests show it at once.)
   auto issue_w = [&](u32 s) {
     const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * T::SB;
     const u32 wl = lds_w + (s & 1u) * kWStageBytes;
