@@ -209,13 +209,14 @@ __device__ __forceinline__ void finish_tiles(const f32x16 (&tot)[NT], float* __r
         }
     return;
   }
-  // The parts cross workgroups (and XCDs): 16-byte buffer accesses at agent scope (sc1), a lane's eight sums side
-  // by side:   partial[((part * tiles + tile) * strips + strip) * 64 + lane][8]
+  // The parts cross workgroups (and XCDs): 16-byte buffer accesses at agent scope (sc1); a wave's tokens 0..7 of the
+  // tile as one KB (lane l at 16 l), its tokens 8..15 as the next, so that a store instruction writes whole lines:
+  //   partial[((part * tiles + tile) * strips + strip)][2][64 lanes][4]
   u32* counters = reinterpret_cast<u32*>(ws);
   const u32 strips = groups * waves;
   const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       ws + kCounterBytes, 0, static_cast<int>(static_cast<size_t>(kparts) * tiles * strips * 2048u), 0x00020000);
-  auto slot_of = [&](u32 pt, u32 tile) { return static_cast<int>((((pt * tiles + tile) * strips + strip) * 64u + lane) * 32u); };
+  auto slot_of = [&](u32 pt, u32 tile) { return static_cast<int>(((pt * tiles + tile) * strips + strip) * 2048u + lane * 16u); };
   bool lower[NT], upper[NT];      // tokens 0..7 / 8..15 of the tile exist (val[0..3] / val[4..7])
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -227,7 +228,7 @@ __device__ __forceinline__ void finish_tiles(const f32x16 (&tot)[NT], float* __r
                                              part_rsrc, slot_of(part, tile), 0, 16);
     if (upper[t])
       __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(val[t][4]), __float_as_uint(val[t][5]), __float_as_uint(val[t][6]), __float_as_uint(val[t][7])},
-                                             part_rsrc, slot_of(part, tile) + 16, 0, 16);
+                                             part_rsrc, slot_of(part, tile) + 1024, 0, 16);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the coherent stores have been acknowledged
   asm volatile("s_barrier" ::: "memory");
@@ -258,7 +259,7 @@ __device__ __forceinline__ void finish_tiles(const f32x16 (&tot)[NT], float* __r
         for (u32 pp = 0; pp < W; ++pp) {
           const u32 pt = min(p0 + pp, kparts - 1u);
           lo[t][pp] = lower[t] ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt, tg * NT + t), 0, 16) : u32x4{0u, 0u, 0u, 0u};
-          hi[t][pp] = upper[t] ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt, tg * NT + t) + 16, 0, 16) : u32x4{0u, 0u, 0u, 0u};
+          hi[t][pp] = upper[t] ? __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, slot_of(pt, tg * NT + t) + 1024, 0, 16) : u32x4{0u, 0u, 0u, 0u};
         }
 #pragma unroll
       for (int t = 0; t < NT; ++t)

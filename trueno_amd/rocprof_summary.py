@@ -6,6 +6,14 @@
       HBM bytes per launch of one kernel from two counter runs (`--pmc FETCH_SIZE`, `--pmc WRITE_SIZE`, KiB per
       dispatch), each scaled by what the same counter reads for the 256 MiB kq_copy_u128 of the same run; with --json the
       figure bench.py reports as `roofline.traffic` is written, stamped with the commit of the working tree.
+  python -m trueno_amd.rocprof_summary shapes <fetch_dir> <write_dir> [--prefix q4k_gemm]
+      the same two counters per kernel and launch shape (a Markdown table): for kernels that serve several shapes
+  python -m trueno_amd.rocprof_summary runs <trace_dir> [<fetch_dir> <write_dir>] [--prefix q4k_gemm] [--min 100]
+      runs of consecutive dispatches of one kernel and launch shape, in the order of the program (bench.py times a
+      configuration as one such run: 20 + 5 x 200 launches over distinct copies, then as many on one copy): calls and
+      average duration per run, with the two counters per run when their directories are given
+  python -m trueno_amd.rocprof_summary pmc <dir> [--prefix q4k_gemm] [--min 100]
+      every counter of one `--pmc` run, averaged per dispatch over the same runs of consecutive dispatches
 
 The runs (on the GPU box, `cd /tmp && export TMPDIR=/tmp` first):
   rocprofv3 --kernel-trace --stats -d <dir> -- python3 bench.py --steps 10 --warmup 2 --no-cpu-baseline --no-executors --no-configs
@@ -80,6 +88,88 @@ def traffic(fetch_dir: str, write_dir: str, kernel: str, json_out: str | None) -
             f.write("\n")
 
 
+def shapes(fetch_dir: str, write_dir: str, prefix: str) -> None:
+    def table(path, counter):
+        out = {}
+        for db in _dbs(path):
+            con = sqlite3.connect(db)
+            q = ("select kernel_name, grid_size_x, workgroup_size_x, avg(value), count(*) from counters_collection "
+                 "where counter_name = ? group by kernel_name, grid_size_x, workgroup_size_x")
+            for name, grid, wg, avg, n in con.execute(q, (counter,)):
+                out[(name.split("(")[0], grid, wg)] = (float(avg), int(n))
+        return out
+    fetch, write = table(fetch_dir, "FETCH_SIZE"), table(write_dir, "WRITE_SIZE")
+    copy_f = [v[0] for k, v in fetch.items() if k[0] == COPY_KERNEL]
+    copy_w = [v[0] for k, v in write.items() if k[0] == COPY_KERNEL]
+    if not copy_f or not copy_w:
+        raise SystemExit(f"need a dispatch of {COPY_KERNEL} in both runs")
+    scale_f, scale_w = COPY_KIB / copy_f[0], COPY_KIB / copy_w[0]
+    print(f"scale: fetch {scale_f:.4f}, write {scale_w:.4f} ({COPY_KERNEL} over 256 MiB: FETCH_SIZE {copy_f[0]:.1f} KiB, WRITE_SIZE {copy_w[0]:.1f} KiB)")
+    print("| kernel | grid threads | block | dispatches | FETCH KiB raw | WRITE KiB raw | HBM bytes (scaled) |")
+    print("|---|---|---|---|---|---|---|")
+    for key in sorted(fetch):
+        if not key[0].startswith(prefix) or key not in write:
+            continue
+        f, w = fetch[key], write[key]
+        print(f"| {key[0]} | {key[1]} | {key[2]} | {f[1]} | {f[0]:.1f} | {w[0]:.1f} | {round((f[0] * scale_f + w[0] * scale_w) * 1024):,} |")
+
+
+def _runs(path: str, query: str, prefix: str):
+    """[(key, [values])] for consecutive rows with the same key = (kernel, grid, block)"""
+    out = []
+    for db in _dbs(path):
+        con = sqlite3.connect(db)
+        for name, grid, wg, value in con.execute(query):
+            key = (name.split("(")[0], grid, wg)
+            if out and out[-1][0] == key:
+                out[-1][1].append(float(value))
+            else:
+                out.append((key, [float(value)]))
+    return [(k, v) for k, v in out if k[0].startswith(prefix)]
+
+
+def runs(trace_dir: str, fetch_dir: str | None, write_dir: str | None, prefix: str, least: int) -> None:
+    tr = [r for r in _runs(trace_dir, "select name, grid_x, workgroup_x, end - start from kernels order by start", prefix)
+          if len(r[1]) >= least]
+    cols = [tr]
+    if fetch_dir and write_dir:
+        q = ("select kernel_name, grid_size_x, workgroup_size_x, value from counters_collection where counter_name = '{}' "
+             "order by dispatch_id")
+        fetch = [r for r in _runs(fetch_dir, q.format("FETCH_SIZE"), prefix) if len(r[1]) >= least]
+        write = [r for r in _runs(write_dir, q.format("WRITE_SIZE"), prefix) if len(r[1]) >= least]
+        if [r[0] for r in fetch] != [r[0] for r in tr] or [r[0] for r in write] != [r[0] for r in tr]:
+            raise SystemExit("the three runs do not show the same sequence of kernel runs")
+        copy_f = _runs(fetch_dir, q.format("FETCH_SIZE"), COPY_KERNEL)[0][1][0]
+        copy_w = _runs(write_dir, q.format("WRITE_SIZE"), COPY_KERNEL)[0][1][0]
+        print(f"scale: fetch {COPY_KIB / copy_f:.4f}, write {COPY_KIB / copy_w:.4f}")
+        cols += [fetch, write, COPY_KIB / copy_f, COPY_KIB / copy_w]
+    head = "| # | kernel | grid threads | block | calls | average us | min us |"
+    print(head + (" FETCH KiB raw | WRITE KiB raw | HBM bytes (scaled) |" if len(cols) > 1 else ""))
+    print("|---" * (head.count("|") - 1 + (3 if len(cols) > 1 else 0)) + "|")
+    for i, (key, d) in enumerate(tr):
+        line = f"| {i} | {key[0]} | {key[1]} | {key[2]} | {len(d)} | {sum(d) / len(d) / 1e3:.2f} | {min(d) / 1e3:.2f} |"
+        if len(cols) > 1:
+            f, w = cols[1][i][1], cols[2][i][1]
+            fa, wa = sum(f) / len(f), sum(w) / len(w)
+            line += f" {fa:.1f} | {wa:.1f} | {round((fa * cols[3] + wa * cols[4]) * 1024):,} |"
+        print(line)
+
+
+def pmc(path: str, prefix: str, least: int) -> None:
+    names = []
+    for db in _dbs(path):
+        names += [r[0] for r in sqlite3.connect(db).execute("select distinct counter_name from counters_collection order by 1")]
+    names = sorted(set(names))
+    q = ("select kernel_name, grid_size_x, workgroup_size_x, value from counters_collection where counter_name = '{}' "
+         "order by dispatch_id")
+    tables = [[r for r in _runs(path, q.format(n), prefix) if len(r[1]) >= least] for n in names]
+    print("| # | kernel | grid threads | block | calls | " + " | ".join(names) + " |")
+    print("|---" * (5 + len(names)) + "|")
+    for i, (key, d) in enumerate(tables[0]):
+        vals = " | ".join(f"{sum(t[i][1]) / len(t[i][1]):,.0f}" for t in tables)
+        print(f"| {i} | {key[0]} | {key[1]} | {key[2]} | {len(d)} | {vals} |")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -90,9 +180,29 @@ def main() -> int:
     tf.add_argument("write_dir")
     tf.add_argument("--kernel", default="kq_gemv_group")
     tf.add_argument("--json")
+    sh = sub.add_parser("shapes")
+    sh.add_argument("fetch_dir")
+    sh.add_argument("write_dir")
+    sh.add_argument("--prefix", default="")
+    rn = sub.add_parser("runs")
+    rn.add_argument("trace_dir")
+    rn.add_argument("fetch_dir", nargs="?")
+    rn.add_argument("write_dir", nargs="?")
+    rn.add_argument("--prefix", default="")
+    rn.add_argument("--min", type=int, default=100)
+    pm = sub.add_parser("pmc")
+    pm.add_argument("dir")
+    pm.add_argument("--prefix", default="")
+    pm.add_argument("--min", type=int, default=100)
     a = ap.parse_args()
     if a.cmd == "trace":
         trace(a.dir)
+    elif a.cmd == "pmc":
+        pmc(a.dir, a.prefix, a.min)
+    elif a.cmd == "runs":
+        runs(a.trace_dir, a.fetch_dir, a.write_dir, a.prefix, a.min)
+    elif a.cmd == "shapes":
+        shapes(a.fetch_dir, a.write_dir, a.prefix)
     else:
         traffic(a.fetch_dir, a.write_dir, a.kernel, a.json)
     return 0
