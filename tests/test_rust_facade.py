@@ -1,7 +1,8 @@
 """The Rust binding under rust/trueno-gpu-hip is source only (no Rust toolchain in this image): these checks keep it
 in step with the C header it binds - every exported function declared with the same number of parameters, the
 constants with the same values, trn_gemv_desc with the same fields in the same order, and the CudaDriver table of
-`src/sys.rs` loading the symbols INTEGRATION.md lists for the reference's 25 `cu*` fields."""
+`src/sys.rs` holding the reference's 25 `cu*` fields (trueno-gpu/src/driver/sys.rs:99-201), each loaded from its
+`trn_*` symbol."""
 import os
 import re
 
@@ -59,11 +60,25 @@ def test_gemv_desc_layout():
     assert "#[repr(C)]" in FFI.split("pub struct trn_gemv_desc")[0][-80:]
 
 
-def test_driver_table_binds_the_symbols_of_the_integration_guide():
-    guide = open(os.path.join(ROOT, "INTEGRATION.md")).read()
-    rows = re.findall(r"\| `(cu\w+)` \(:\d+\) \| `(trn_\w+)`", guide)
-    assert len(rows) == 25
-    for field, symbol in rows:
+# the reference's table, in its order, and the symbol that fills each field
+DRIVER_TABLE = [
+    ("cuInit", "trn_init"), ("cuDeviceGetCount", "trn_device_get_count"), ("cuDeviceGet", "trn_device_get"),
+    ("cuDeviceGetName", "trn_device_get_name"), ("cuDeviceTotalMem", "trn_device_total_mem"),
+    ("cuDevicePrimaryCtxRetain", "trn_primary_ctx_retain"), ("cuDevicePrimaryCtxRelease", "trn_primary_ctx_release"),
+    ("cuCtxSetCurrent", "trn_ctx_set_current"), ("cuCtxSynchronize", "trn_ctx_synchronize"),
+    ("cuModuleLoadData", "trn_module_load_data"), ("cuModuleUnload", "trn_module_unload"),
+    ("cuModuleGetFunction", "trn_module_get_function"), ("cuMemAlloc", "trn_mem_alloc"), ("cuMemFree", "trn_mem_free"),
+    ("cuMemcpyHtoD", "trn_memcpy_htod"), ("cuMemcpyDtoH", "trn_memcpy_dtoh"), ("cuMemcpyHtoDAsync", "trn_memcpy_htod_async"),
+    ("cuMemcpyDtoHAsync", "trn_memcpy_dtoh_async"), ("cuMemcpyDtoD", "trn_memcpy_dtod"),
+    ("cuMemcpyDtoDAsync", "trn_memcpy_dtod_async"), ("cuMemGetInfo", "trn_mem_get_info"),
+    ("cuStreamCreate", "trn_stream_create"), ("cuStreamDestroy", "trn_stream_destroy"),
+    ("cuStreamSynchronize", "trn_stream_synchronize"), ("cuLaunchKernel", "trn_launch_kernel"),
+]
+
+
+def test_driver_table_holds_the_reference_fields_and_binds_exported_symbols():
+    assert len(DRIVER_TABLE) == 25
+    for field, symbol in DRIVER_TABLE:
         assert re.search(rf"pub {field}:\s*unsafe extern \"C\" fn", SYS), field
         assert re.search(rf"{field}: sym!\(b\"{symbol}\\0\"\)", SYS), (field, symbol)
     exported = _c_functions()
