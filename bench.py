@@ -6,15 +6,18 @@ A step is one 7B-style decode weight pass: 32 layers x {Q,K,V,O: Q4_K 4096x4096;
 distinct, seeded synthetic weights resident in HBM (far beyond the 256 MB Infinity Cache, so every
 pass streams from HBM).  Data flow, per layer: a fresh x_l ~ N(0,1) feeds q, k, v, gate and up; o
 consumes the RMS-normalised output of q; down consumes the RMS-normalised output of gate; the head
-consumes the RMS-normalised output of the last down.  The list (trueno_amd.decode_pass, the one the
-GPU parity test checks) goes to the library in one call, in layer order (trn_kquant_gemv_batch).
+consumes the RMS-normalised output of the last down.  Every layer writes activation buffers of its own,
+so nothing but that data flow orders the entries (with one set of buffers shared by all layers, as a
+decoder's are, a layer's q must also wait until the previous layer's o has read it: that pass is timed
+too, `same_pass_with_shared_activation_buffers` in `config`).  The list (trueno_amd.decode_pass, the one
+the GPU parity test checks) goes to the library in one call, in layer order (trn_kquant_gemv_batch).
 `value` is algorithmic bytes (weights + x + y, each once) over wall time.  After the timed region the
 last layer's outputs and the logits are checked against fp64 on their actual inputs.  The same 225
 GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate;
 h <- down) are timed too: `strict_decoder_chain` in `config`.
 
 Prints one JSON line.  `roofline`: the dominant kernel (kq_gemv_group: the launches that carry several
-independent entries, 64 per pass, 3.99 of the 4.13 GB), its launches of one pass timed with HIP events on
+independent entries, 28 per pass, 3.99 of the 4.13 GB), its launches of one pass timed with HIP events on
 their stream, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other
 benchmark configurations, timed as launches back to back over at least 1 GiB of distinct copies
@@ -44,8 +47,8 @@ TRAFFIC_JSON = os.path.join(ROOT, "profiles", "kquant_gemv_group_traffic.json")
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10, help="untimed passes first (the clocks take some ten milliseconds of load to settle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the tables of configurations 1, 2, 3 and 5 and of the path's neighbours")
     ap.add_argument("--no-executors", action="store_true", help="skip the comparison run of the opt-in one-launch executor")
@@ -90,7 +93,8 @@ def main() -> int:
     y = {n: t.GpuBuffer(ctx, n, np.float32) for n in (4096, 11008, 14336, 32000)}
     print(f"[bench] generated and uploaded {layers} layers in {time.time() - t_gen:.1f} s", file=sys.stderr, flush=True)
 
-    batch, strict_batch, layer_batch = dp.build("fresh_x"), dp.build("strict"), dp.build("folded")
+    batch, shared_batch = dp.build("fresh_x_own_buffers"), dp.build("fresh_x")
+    strict_batch, layer_batch = dp.build("strict"), dp.build("folded")
     entry_bytes, entry_names = dp.entry_bytes(), dp.entry_names()
     total_bytes, weight_bytes = sum(entry_bytes), dp.weight_bytes()
     act, logits, head_w = dp.act, dp.logits, dp.head_w
@@ -134,13 +138,12 @@ def main() -> int:
     ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- what the timed passes left behind, against fp64 on the actual inputs: the last layer (whose outputs are still
-    #      in the shared activation buffers) and the logits ----------------------------------------------------------
+    # ---- what the timed passes left behind, against fp64 on the actual inputs: the last layer and the logits ------
     def norm64(v, eps=1e-6):
         v = v.astype(np.float64)
         return v / np.sqrt(np.mean(v * v) + eps)
 
-    got = {nm: b.copy_to_host() for nm, b in act.items()}
+    got = {nm: b.copy_to_host() for nm, b in dp.act_of_layer[layers - 1].items()}
     got["logits"] = logits.copy_to_host()
     x_last = xs[layers - 1].astype(np.float64)
     inputs = {"q": x_last, "k": x_last, "v": x_last, "gate": x_last, "up": x_last, "o": norm64(got["q"]), "down": norm64(got["gate"])}
@@ -217,6 +220,16 @@ def main() -> int:
     if not args.pass_only:
         strict_ms, _ = run_passes(max(3, args.steps // 2), 2, strict_batch)
         layer_ms, _ = run_passes(max(3, args.steps // 2), 2, layer_batch)
+
+    # ---- the same pass with ONE set of activation buffers shared by all layers, as a decoder's are: the write-after-
+    #      read hazards between layers cut it into more, smaller launches.  Same logits, bit for bit. ----------------
+    shared = None
+    if not args.pass_only:
+        shared_ms, _ = run_passes(max(3, args.steps // 2), 2, shared_batch)
+        assert np.array_equal(logits.copy_to_host().view(np.uint32), got["logits"].view(np.uint32)), \
+            "the pass with shared activation buffers must give the headline pass's logits"
+        shared = {"us_per_pass": round(shared_ms * 1e3, 1), "gbps": round(total_bytes / shared_ms / 1e6, 1),
+                  "frac_of_hbm_peak": round(total_bytes / shared_ms / 1e6 / HBM_PEAK_GBPS, 4), "launches": max(shared_batch.plan()) + 1}
 
     # ---- the same list through the one-launch executor (opt-in), for comparison ------------------------
     other_modes = {}
@@ -478,12 +491,15 @@ def main() -> int:
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"7B-style decode weight pass: {layers} layers x (4x Q4_K 4096x4096 + 2x Q4_K 11008x4096 + "
                                f"1x Q6_K 4096x11008) + Q6_K 32000x4096 head; {len(batch)} GEMVs in layer order "
-                               f"(per layer x_l~N(0,1) -> q,k,v,gate,up; o<-norm(q); down<-norm(gate); head<-norm(down)), "
+                               f"(per layer x_l~N(0,1) -> q,k,v,gate,up; o<-norm(q); down<-norm(gate); head<-norm(down); "
+                               f"activation buffers per layer), "
                                f"{total_bytes / 1e9:.3f} GB, batch 1, f32 x and y", "gemvs": len(batch),
                    "bytes_per_step": total_bytes, "launches_per_step": max(launch_of) + 1,
                    # the same matrices in the data flow of a real decoder: every step waits for the one before it
                    "strict_decoder_chain": chain(strict_ms) and dict(chain(strict_ms), dependent_steps=max(strict_batch.plan()) + 1),
-                   "strict_decoder_chain_with_folded_layer_glue": chain(layer_ms)},
+                   "strict_decoder_chain_with_folded_layer_glue": chain(layer_ms),
+                   # the headline's data flow with one set of activation buffers for all layers (more, smaller launches)
+                   "same_pass_with_shared_activation_buffers": shared},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic["bytes_per_launch"] if traffic else None,

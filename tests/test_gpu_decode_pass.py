@@ -84,3 +84,23 @@ def test_bench_list_default_mode(gpu, decode_pass, flow):
         err = kq.rel_l2(got[nm], ref)
         print(f"  {flow} {nm}: rel-L2 {err:.2e}", flush=True)
         assert err <= TOL, (flow, nm, err)
+
+
+def test_buffers_per_layer_give_the_same_bits_in_fewer_launches(gpu, decode_pass):
+    """The same data flow with activation buffers of its own for every layer: the library brings independent entries
+    of neighbouring layers together, and every layer's outputs and the logits are those of the shared-buffer pass
+    (whose last layer is still in its buffers), bit for bit."""
+    ctx, stream = gpu
+    p = decode_pass[0]
+    shared = p.build("fresh_x")
+    shared.launch(stream)
+    stream.synchronize()
+    want = _snapshot(p)
+    own = p.build("fresh_x_own_buffers")
+    assert max(own.plan()) < max(shared.plan()), (own.plan(), shared.plan())
+    p.logits.copy_from_host(np.zeros(HEAD[2], np.float32))
+    own.launch(stream)
+    stream.synchronize()
+    assert np.array_equal(p.logits.copy_to_host().view(np.uint32), want["logits"].view(np.uint32))
+    for nm, b in p.act_of_layer[LAYERS - 1].items():
+        assert np.array_equal(b.copy_to_host().view(np.uint32), want[nm].view(np.uint32)), nm

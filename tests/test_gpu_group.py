@@ -16,7 +16,7 @@ def _tune(key, value):
     assert _ffi.lib().trn_set_tuning(key.encode(), int(value)) == 0
 
 
-def _run(gpu, specs, x_len, group_off):
+def _run(gpu, specs, x_len, group_off, plan_out=None):
     ctx, stream = gpu
     host = {"x": kq.gen_x(1, x_len)}
     bufs = {"x": t.GpuBuffer.from_host(ctx, host["x"])}
@@ -31,6 +31,8 @@ def _run(gpu, specs, x_len, group_off):
         batch.add(fmt, k, n, bufs[dst], w, bufs[src], flags)
     _tune("group_off", group_off)
     try:
+        if plan_out is not None:
+            plan_out.extend(batch.plan())
         batch.launch(stream)
         stream.synchronize()
     finally:
@@ -74,6 +76,34 @@ def test_grouped_equals_separate(gpu, case):
         if flags:
             ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
         assert kq.rel_l2(got[dst], ref) <= TOL, (case, dst)
+
+
+@pytest.mark.parametrize("group_max", (0, 11, 16))
+def test_up_to_sixteen_entries_in_one_launch(gpu, group_max):
+    """Nineteen independent entries of mixed formats and shapes: by default eight to a launch; with "group_max" raised a
+    launch holds up to sixteen (every position of the kernel's table of first workgroups is used).  Same bits as one
+    launch per entry."""
+    fmts = ("q4k", "q5k", "q6k")
+    specs = [(fmts[i % 3], 33 + 41 * i, 256 * (1 + (i * 5) % 7), "x", f"y{i}", i % 2) for i in range(19)]
+    sep, _ = _run(gpu, specs, 256 * 7, 1)
+    _tune("group_max", group_max)
+    _tune("group_window", 32)
+    plan = []
+    try:
+        got, mats = _run(gpu, specs, 256 * 7, 0, plan)
+    finally:
+        _tune("group_max", 0)
+        _tune("group_window", 0)
+    most = {0: 8, 11: 11, 16: 16}[group_max]
+    assert len(plan) == 19 and max(np.bincount(plan)) == most and max(plan) + 1 == -(-19 // most), plan
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), (group_max, name)
+    for (fmt, n, k, src, dst, flags), m in zip(specs, mats):
+        x = got[src][:k].astype(np.float64)
+        ref = kq.dequant_matrix(fmt, m, n, k).astype(np.float64) @ x
+        if flags:
+            ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
+        assert kq.rel_l2(got[dst], ref) <= TOL, (group_max, dst)
 
 
 @pytest.mark.parametrize("seed", (0, 1, 2, 3))

@@ -87,9 +87,9 @@ KQ_GEMV_KERNELS(q4k, FMT_Q4K)
 KQ_GEMV_KERNELS(q5k, FMT_Q5K)
 KQ_GEMV_KERNELS(q6k, FMT_Q6K)
 
-// Up to eight GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
-// up) in one launch: consecutive runs of workgroups belong to consecutive entries.  Each entry is computed
-// exactly as its own launch would compute it.
+// Up to sixteen GEMVs that do not depend on one another (the q, k, v projections of a decoder layer; gate and
+// up; entries of neighbouring layers where a list allows it) in one launch: consecutive runs of workgroups belong to
+// consecutive entries.  Each entry is computed exactly as its own launch would compute it.
 // A workgroup can ask for its first rows only once it knows its matrix, and kernel arguments come from memory: finding
 // the entry through a table in the argument and then reading the entry would be two memory round trips in a row.  The
 // table therefore travels as eight leading scalar arguments, which the build asks the hardware to place in scalar
@@ -99,6 +99,7 @@ struct GemvGroupHot {
   const uint8_t* w;
   const float* x;
   u32 k, n, fmt, flags;
+  u32 first_block, num_blocks;      // the entry's run of workgroups
 };
 struct GemvGroupCold {
   float* y;
@@ -108,27 +109,36 @@ struct GemvGroupCold {
   float eps;
   u32 pad;
 };
+constexpr u32 kGroupEntries = 16;
 struct GemvGroup {
-  GemvGroupHot hot[8];
-  GemvGroupCold cold[8];
+  GemvGroupHot hot[kGroupEntries];
+  GemvGroupCold cold[kGroupEntries];
 };
-// first1 .. first8: first[j] is the first workgroup of entry j (first[0] = 0; entries that do not exist repeat the grid size)
+// firsts: first[j], j = 1 .. 16, is the first workgroup of entry j (entries that do not exist, and first[16], repeat the
+// grid size), two to an argument: first[2a + 1] in the low half of argument a, first[2a + 2] in the high half (a grid has
+// fewer than 65536 workgroups).  The entry of a workgroup is the last one that starts at or before it: four compares.
 extern "C" __global__ void __launch_bounds__(768)
-kq_gemv_group(u32 first1, u32 first2, u32 first3, u32 first4, u32 first5, u32 first6, u32 first7, u32 first8, const GemvGroup g) {
+kq_gemv_group(u32 firsts0, u32 firsts1, u32 firsts2, u32 firsts3, u32 firsts4, u32 firsts5, u32 firsts6, u32 firsts7, const GemvGroup g) {
   extern __shared__ f32x4 lds4[];
   __shared__ u32 s_flag;
-  const u32 fr[9] = {0u, first1, first2, first3, first4, first5, first6, first7, first8};
-  u32 i = 0, wg0 = fr[0], wg1 = fr[1];
-#pragma unroll
-  for (u32 j = 1; j < 8; ++j)
-    if (blockIdx.x >= fr[j]) { i = j; wg0 = fr[j]; wg1 = fr[j + 1]; }       // first[] never decreases
+  const u32 b = blockIdx.x;
+  u32 i = b >= (firsts3 >> 16) ? 8u : 0u;                                               // first[8]
+  i += b >= ((i ? firsts5 : firsts1) >> 16) ? 4u : 0u;                                  // first[12], first[4]
+  const u32 p2 = (i & 8u) ? ((i & 4u) ? firsts6 : firsts4) : ((i & 4u) ? firsts2 : firsts0);      // first[i + 2]
+  i += b >= (p2 >> 16) ? 2u : 0u;
+  // first[i + 1]: the low half of argument i / 2, picked bit by bit (selects, no branches)
+  const u32 q0 = (i & 8u) ? firsts4 : firsts0, q1 = (i & 8u) ? firsts5 : firsts1, q2 = (i & 8u) ? firsts6 : firsts2,
+            q3 = (i & 8u) ? firsts7 : firsts3;
+  const u32 r0 = (i & 4u) ? q2 : q0, r1 = (i & 4u) ? q3 : q1;
+  const u32 p1 = (i & 2u) ? r1 : r0;
+  i += b >= (p1 & 0xFFFFu) ? 1u : 0u;
   GemvGroupHot h = g.hot[i];
   const GemvGroupCold c = g.cold[i];
   // the block size is an implicit kernel argument, a load like the entry's: all of them in flight together, one wait
   u32 block_threads = blockDim.x;
   asm volatile("" : "+s"(block_threads), "+s"(h.k), "+s"(h.flags));
   const ChainEntry e = {h.fmt, h.k, h.n, h.flags, h.w, h.x, c.y, c.gamma, c.x2, c.residual, c.eps, 0u};
-  const u32 block_id = blockIdx.x - wg0, num_blocks = wg1 - wg0;
+  const u32 block_id = b - h.first_block, num_blocks = h.num_blocks;
   if (e.fmt == FMT_Q4K) chain_step<FMT_Q4K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
   else if (e.fmt == FMT_Q5K) chain_step<FMT_Q5K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
   else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);

@@ -97,7 +97,7 @@ std::atomic<int> g_tune_gemm_tiles{0};      // token tiles per workgroup of the 
 std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 std::atomic<int> g_tune_attention_min_steps{0};
 std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped launch may look ahead over (0: 16)
-std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8)
+std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8; at most 16)
 std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
 std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
@@ -609,7 +609,12 @@ uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u +
 // batch_mode 1: the list as phases of independent entries in ONE resident launch (kq_gemv_phases): one workgroup
 // of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
 // barrier between phases.  *handled = false (and hipSuccess): not possible here, issue the list the plain way.
-constexpr uint32_t kGroupMax = 8;      // entries of one grouped launch
+constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (kGroupEntries of the kernel)
+// Entries a launch takes by default.  More is not better: on the 7B pass with activation buffers per layer, launches of
+// 8 entries (138 MB, 30 launches) take 880 us, of 12 entries 940 us, of 16 entries (275 MB, 16 launches) 1075-1095 us - with
+// more entries each one's share of the workgroups gets coarse (9 of 256 for a 4096 x 4096 matrix beside a 4096 x 11008
+// one) and the launch ends as unevenly.
+constexpr uint32_t kGroupDefault = 8;
 bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
   return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
          gemv_geometry(*dk, d.k, d.n).fits;
@@ -621,9 +626,9 @@ bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
 // overtake.  What an entry computes does not depend on the company it is launched in, so the results are those of
 // the list in order.
 void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches) {
-  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 16u);
+  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 2u * kGroupDefault);
   const uint32_t group_max =
-      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupMax);
+      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupDefault);
   std::vector<uint8_t> launched(count, 0);
   for (uint32_t pos = 0; pos < count;) {
     if (launched[pos]) { ++pos; continue; }
@@ -1240,10 +1245,10 @@ trn_status trn_q6k_gemm(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c, uint32
 
 namespace {
 struct GemvGroupHost {   // GemvGroup of kquant_kernels.hip: what a workgroup's first loads need, then the rest
-  struct Hot { uint64_t w, x; uint32_t k, n, fmt, flags; } hot[kGroupMax];
+  struct Hot { uint64_t w, x; uint32_t k, n, fmt, flags, first_block, num_blocks; } hot[kGroupMax];
   struct Cold { uint64_t y, gamma, x2, residual; float eps; uint32_t pad; } cold[kGroupMax];
 };
-static_assert(sizeof(GemvGroupHost) == kGroupMax * (32 + 40), "GemvGroup layout");
+static_assert(sizeof(GemvGroupHost) == kGroupMax * (40 + 40), "GemvGroup layout");
 
 bool gemv_depends(const trn_gemv_desc& g, const trn_gemv_desc& p) { return desc_conflict(g, p); }
 
@@ -1281,7 +1286,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     const double bytes = cost_of(e);
     const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
     const uint64_t x_bytes = uint64_t(e.k) * 4u;
-    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags};
+    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags, 0u, 0u};
     g.cold[i] = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
     // workgroups of 8 waves or more hand their row batches out among the waves: a share need not be a whole
     // number of rounds of all waves
@@ -1294,9 +1299,14 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     const uint32_t grid = uint32_t((uint64_t(e.n) + rows - 1) / rows);
     lds = std::max<uint32_t>(lds, uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch));
     first[i + 1] = first[i] + grid;
+    g.hot[i].first_block = first[i];
+    g.hot[i].num_blocks = grid;
   }
   for (uint32_t i = len; i < kGroupMax; ++i) first[i + 1] = first[len];   // entries that do not exist own no workgroup
-  void* args[] = {&first[1], &first[2], &first[3], &first[4], &first[5], &first[6], &first[7], &first[8], &g};
+  if (first[len] > 0xFFFFu) return hipErrorInvalidValue;                  // the table holds 16 bits per entry
+  uint32_t packed[8];
+  for (uint32_t a = 0; a < 8; ++a) packed[a] = first[2 * a + 1] | first[2 * a + 2] << 16;
+  void* args[] = {&packed[0], &packed[1], &packed[2], &packed[3], &packed[4], &packed[5], &packed[6], &packed[7], &g};
   return hipModuleLaunchKernel(d->gemv_group, first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
 }
 }  // namespace

@@ -2,9 +2,13 @@
 (Q4_K 4096x4096), gate, up (Q4_K 11008x4096), down (Q6_K 4096x11008), then the Q6_K 32000x4096 head.  The benchmark and
 the parity tests build their lists here, so what is timed is what is checked.
 
-Three ways of wiring the same matrices (`flow`):
+Four ways of wiring the same matrices (`flow`):
   "fresh_x"  a given vector x_l per layer feeds q, k, v, gate, up; o reads the RMS-normalised output of q, down that
-             of gate, the head that of the last down.  Activation buffers are shared by all layers.
+             of gate, the head that of the last down.  Activation buffers are shared by all layers, as a decoder's
+             are: a layer's q may only be written once the previous layer's o has read it.
+  "fresh_x_own_buffers"  the same data flow with activation buffers of its own for every layer: nothing but o <- q and
+             down <- gate inside a layer (and head <- the last down) orders the entries, so independent entries of
+             neighbouring layers fill the launches.  Same results as "fresh_x", bit for bit.
   "strict"   the serial data flow of a decoder: q, k, v <- h; o <- q; gate, up <- o; down <- gate; h <- down,
              every input RMS-normalised (129 dependent steps).
   "folded"   the decoder layer with its element-wise steps folded into the entries: q, k, v <- rmsnorm(h) * g1;
@@ -40,6 +44,7 @@ class DecodePass:
         self.logits = GpuBuffer(ctx, HEAD[2], np.float32)
         self.res = None
         self.gammas = None
+        self.act_of_layer = None
 
     def entry_names(self):
         return [name for _ in range(self.layers) for name, _, _, _ in LAYER_MATS] + ["head"]
@@ -67,6 +72,17 @@ class DecodePass:
                     b.add(fmt, k, n, act[name], self.weights[layer][name], x, flags)
                 h = act["down"]
             b.add(HEAD[1], HEAD[3], HEAD[2], self.logits, self.head_w, act["down"], NORM)
+            return b
+        if flow == "fresh_x_own_buffers":
+            if self.act_of_layer is None:
+                self.act_of_layer = [{nm: GpuBuffer(self.ctx, n, np.float32) for nm, n in ACT} for _ in range(self.layers)]
+            for layer in range(self.layers):
+                own = self.act_of_layer[layer]
+                for name, fmt, n, k in LAYER_MATS:
+                    src = {"o": "q", "down": "gate"}.get(name)
+                    x, flags = (self.xs[layer], 0) if src is None else (own[src], NORM)
+                    b.add(fmt, k, n, own[name], self.weights[layer][name], x, flags)
+            b.add(HEAD[1], HEAD[3], HEAD[2], self.logits, self.head_w, self.act_of_layer[-1]["down"], NORM)
             return b
         if flow != "folded":
             raise ValueError(flow)
