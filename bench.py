@@ -168,7 +168,7 @@ def main() -> int:
         members.setdefault(l, []).append(i)
     kinds = {}
     for l in sorted(members):
-        sig = "[" + ",".join(entry_names[i] for i in members[l]) + "]"
+        sig = "[" + ",".join(entry_names[i] for i in members[l]) + "] " + f"{sum(entry_bytes[i] for i in members[l]) / 1e6:.1f} MB"
         kinds[sig] = kinds.get(sig, 0) + 1
     print("[bench] launches of the pass: " + ", ".join(f"{c} x {sig}" for sig, c in kinds.items()), file=sys.stderr, flush=True)
     groups, grp_bytes = [], 0
