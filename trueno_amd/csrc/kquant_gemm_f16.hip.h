@@ -352,7 +352,8 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   // ordinary loads of A the compiler waits for vmcnt(0) wherever DMA is also in flight, which takes the copies of W out
   // of the background.  The price of asm: between such a load and the wait that names its registers the compiler must
   // have no reason to copy them - one definition per loop, no second set of registers joined to the first; a variant
-  // that requested two super-blocks up front broke exactly there, and the parity tests show it at once.)
+  // that requested two super-blocks up front broke exactly there; the build refuses such assembly (check_asm_loads.py) and
+  // the parity tests show it at once.)
   auto issue_w = [&](u32 s) {
     const uint8_t* wsrc = w + static_cast<size_t>(sb0 + s) * T::SB;
     const u32 wl = lds_w + (s & 1u) * kWStageBytes;
