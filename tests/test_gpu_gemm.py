@@ -142,6 +142,19 @@ def test_gemm_many_tokens(gpu, fmt):
     assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
 
 
+@pytest.mark.parametrize("m", (5, 20))
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_few_rows_long_k(gpu, fmt, m):
+    """96 rows against K = 8192: one group of strips, so the library cuts K into as many parts as there are
+    super-blocks (32) and the last workgroup adds them in two rounds of sixteen."""
+    n, k = 96, 8192
+    buf, a = kq.gen_matrix(fmt, 300 + m, n, k), kq.gen_x(310 + m, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
+    again = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert np.array_equal(again.view(np.uint32), c.view(np.uint32))
+
+
 @pytest.mark.parametrize("fmt", MFMA_FORMATS)
 def test_gemm_parts_of_k(gpu, fmt):
     """However K is cut into parts the result stays within tolerance, and the same cut gives the same bits on
