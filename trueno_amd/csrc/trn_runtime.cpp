@@ -435,7 +435,8 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   // the counters sit at the front of a region that only grows, so a larger product finds zeros there too (the
   // kernel puts every counter it used back to zero)
   const size_t cnt_cap = kGemmCounterBytes, need = cnt_cap + part_bytes;
-  if (cnt_bytes > cnt_cap) return hipErrorInvalidValue;
+  // (the kernel addresses the parts with 32-bit offsets; a cut by the estimate stays far below that, a forced one may not)
+  if (cnt_bytes > cnt_cap || part_bytes >= (size_t(1) << 32)) return hipErrorInvalidValue;
   uint64_t cnt = ext_base;
   if (ext_base != 0) {
     if (need > ext_cap) return hipErrorInvalidValue;
