@@ -155,6 +155,42 @@ def test_gemm_few_rows_long_k(gpu, fmt, m):
     assert np.array_equal(again.view(np.uint32), c.view(np.uint32))
 
 
+@pytest.mark.parametrize("m", (5, 24, 40))
+def test_gemm_twelve_strips_per_workgroup(gpu, m):
+    """The Q4_K kernel that takes twelve strips of 32 rows per workgroup (its last four waves convert no tokens), forced
+    on a small product whose rows fill neither the last strip nor the last workgroup: within tolerance, and the same
+    bits as eight strips per workgroup for the same cut of K (a strip's sums do not depend on its company)."""
+    n, k = 777, 2048
+    buf, a = kq.gen_matrix("q4k", 400 + m, n, k), kq.gen_x(410 + m, m, k)
+    c64 = _c64("q4k", buf, a, n, k)
+    try:
+        for parts in (1, 3):
+            _tune("gemm_k_parts", parts)
+            _tune("gemm_waves", 12)
+            twelve = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+            assert kq.rel_l2(twelve, c64) <= TOL
+            _tune("gemm_waves", 8)
+            _tune("gemm_tiles", 1)
+            eight = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+            assert np.array_equal(eight.view(np.uint32), twelve.view(np.uint32)), parts
+            _tune("gemm_tiles", 0)
+    finally:
+        _tune("gemm_k_parts", 0)
+        _tune("gemm_waves", 0)
+        _tune("gemm_tiles", 0)
+
+
+@pytest.mark.parametrize("m", (4, 32))
+@pytest.mark.parametrize("fmt", MFMA_FORMATS)
+def test_gemm_ffn_shape_w_11008x4096(gpu, fmt, m):
+    """The 7B gate/up shape: 43 groups of 8 strips do not divide the CUs well, so the library takes fewer parts of K than
+    would fill them (and, for Q4_K with 32 tokens, twelve strips per workgroup)."""
+    n, k = 11008, 4096
+    buf, a = kq.gen_matrix(fmt, 500 + m, n, k), kq.gen_x(510 + m, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
+
+
 @pytest.mark.parametrize("fmt", MFMA_FORMATS)
 def test_gemm_parts_of_k(gpu, fmt):
     """However K is cut into parts the result stays within tolerance, and the same cut gives the same bits on

@@ -300,7 +300,7 @@ struct Geometry {
 // pays when the tokens are many - building them is most of a super-block's instructions.  (finish_tiles: what
 // happens with the results.)
 //   dynamic LDS = lds_bytes(waves, tile bytes, NT)
-template <int FMT, int CHUNKS, int NT>     // CHUNKS: chunks of A a thread converts per super-block and tile, 512 / threads
+template <int FMT, int WAVES, int NT>     // WAVES strips of 32 rows per workgroup (4, 8 or 12): the kernels are launched with 64 * WAVES threads
 __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, uint8_t* __restrict__ ws,
                                          u32 m, u32 n, u32 nsb, uint64_t geom, u32 lds_base) {
   const Geometry cut(geom);
@@ -313,7 +313,9 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   if (unit >= groups * kparts) return;
   const u32 group = unit / kparts, part = unit - group * kparts;
   const u32 sb0 = part * ksb, ns = min(ksb, nsb - sb0);
-  constexpr u32 waves = 8u / CHUNKS;      // the kernels are launched with 512 / CHUNKS threads
+  constexpr u32 waves = WAVES;
+  // chunks of A a thread converts per super-block and tile: 512 over the threads (with 12 waves the last four convert none)
+  constexpr int CHUNKS = WAVES >= 8 ? 1 : 8 / WAVES;
   const u32 strip = group * waves + wave;
   const u32 col = lane & 31u, g = lane >> 5;
   using T = WTile<FMT>;
@@ -333,8 +335,9 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
   const u32 lds_xp = lds_base, lds_w = lds_base + 2u * kStage + wave * (2u * kWStageBytes);
   const u32 lds_flag = lds_base + 2u * kStage + 2u * waves * kWStageBytes;
   // the chunks of A this thread converts per super-block: 512 chunks of 8 elements (16 tokens x 32)
-  constexpr u32 nthreads = 512u / CHUNKS;
+  constexpr u32 nthreads = 64u * WAVES;
   constexpr int NC = CHUNKS * NT;      // chunk i: tile i / CHUNKS of the group
+  const bool converts = WAVES <= 8 || wave < 8u;      // (the others load the same A all the same: one count of loads for every wave)
   const float* asrc[NC];
   u32 ctoken[NC], cpos[NC];
   bool live[NC];
@@ -374,6 +377,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
 #pragma unroll
     for (int i = 0; i < NC; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA) : "memory");
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (!converts) return;
 #pragma unroll
     for (int i = 0; i < NC; ++i)
       convert_chunk(live[i] ? __builtin_bit_cast(f32x4, an[i][0]) : zero4, live[i] ? __builtin_bit_cast(f32x4, an[i][1]) : zero4,

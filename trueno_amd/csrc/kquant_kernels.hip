@@ -292,13 +292,14 @@ KQ_GEMM_KERNELS(q6k, FMT_Q6K)
     gemm_f16::BODY(a, w, c, ws, m, n, nsb, geom, lds_base);                                                              \
   }
 #define KQ_COMMA ,
-KQ_GEMM_F16(q4k_gemm_f16_w8, 512, kq_body<FMT_Q4K KQ_COMMA 1 KQ_COMMA 1>)
-KQ_GEMM_F16(q4k_gemm_f16_w4, 256, kq_body<FMT_Q4K KQ_COMMA 2 KQ_COMMA 1>)
-KQ_GEMM_F16(q5k_gemm_f16_w8, 512, kq_body<FMT_Q5K KQ_COMMA 1 KQ_COMMA 1>)
-KQ_GEMM_F16(q5k_gemm_f16_w4, 256, kq_body<FMT_Q5K KQ_COMMA 2 KQ_COMMA 1>)
+KQ_GEMM_F16(q4k_gemm_f16_w8, 512, kq_body<FMT_Q4K KQ_COMMA 8 KQ_COMMA 1>)
+KQ_GEMM_F16(q4k_gemm_f16_w4, 256, kq_body<FMT_Q4K KQ_COMMA 4 KQ_COMMA 1>)
+KQ_GEMM_F16(q4k_gemm_f16_w12, 768, kq_body<FMT_Q4K KQ_COMMA 12 KQ_COMMA 1>)
+KQ_GEMM_F16(q5k_gemm_f16_w8, 512, kq_body<FMT_Q5K KQ_COMMA 8 KQ_COMMA 1>)
+KQ_GEMM_F16(q5k_gemm_f16_w4, 256, kq_body<FMT_Q5K KQ_COMMA 4 KQ_COMMA 1>)
 // two token tiles per workgroup (more than 16 tokens)
-KQ_GEMM_F16(q4k_gemm_f16_w8t2, 512, kq_body<FMT_Q4K KQ_COMMA 1 KQ_COMMA 2>)
-KQ_GEMM_F16(q5k_gemm_f16_w8t2, 512, kq_body<FMT_Q5K KQ_COMMA 1 KQ_COMMA 2>)
+KQ_GEMM_F16(q4k_gemm_f16_w8t2, 512, kq_body<FMT_Q4K KQ_COMMA 8 KQ_COMMA 2>)
+KQ_GEMM_F16(q5k_gemm_f16_w8t2, 512, kq_body<FMT_Q5K KQ_COMMA 8 KQ_COMMA 2>)
 KQ_GEMM_F16(q6k_gemm_f16_w8, 512, q6k_body<1>)
 KQ_GEMM_F16(q6k_gemm_f16_w4, 256, q6k_body<2>)
 

@@ -77,6 +77,7 @@ struct DeviceKernels {
   hipFunction_t residual_add = nullptr, swiglu = nullptr, rmsnorm = nullptr, residual_rmsnorm = nullptr;
   hipFunction_t gemv_f32_fast = nullptr, gemv_f32_generic = nullptr, q5k_from_ggml = nullptr, attention = nullptr;
   hipFunction_t gemm_f16[NFMT][2] = {};   // [format][4 or 8 strips per workgroup]
+  hipFunction_t gemm_f16_w12 = nullptr;   // Q4_K: 12 strips per workgroup
   hipFunction_t gemm_f16_t2[2] = {};      // Q4_K, Q5_K: 8 strips and two token tiles per workgroup
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
@@ -100,7 +101,7 @@ std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped la
 std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8; at most 16)
 std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
-std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4 or 8 (0: default)
+std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4, 8 or (Q4_K) 12 (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -160,6 +161,7 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.gemm_f16[1][0], "q5k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[1][1], "q5k_gemm_f16_w8")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16_t2[0], "q4k_gemm_f16_w8t2")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_f16_w12, "q4k_gemm_f16_w12")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16_t2[1], "q5k_gemm_f16_w8t2")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][0], "q6k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][1], "q6k_gemm_f16_w8")) != hipSuccess ||
@@ -378,37 +380,60 @@ constexpr size_t kGemmCounterBytes = size_t(1) << 16;   // arrival counters at t
 struct GemmCut { uint32_t waves, nt, groups, tgroups, kparts, ksb; double us; };
 
 // The cut with the least estimated time among: 8 strips and one tile, 8 strips and two tiles (Q4_K and Q5_K: the weight
-// operands are built once for both; the Q6_K kernel has no registers left for it), 4 strips and one tile.  Times in
-// microseconds fitted to measurements on MI355X (Q4_K, 1024 x 4096 .. 14336 x 4096 and 4096 x 14336, 4 .. 512 tokens; they
-// hold within about 15 %): 5 to the first super-block and for the stores (3.5 with 4 strips); a super-block takes a
-// workgroup 2.0 (8 strips), 3.2 (8 strips, two tiles) or 1.5 (4 strips); with K in parts 2.5 for publishing a part, plus the time in
-// which the workgroup that arrives last reads every part of its rows through one CU, at about 40 GB/s - with 16 parts
-// of 8 strips that read alone took 6.5 us of 15 (4096 x 4096, M = 16: 15.0 us with 8 strips, 10.3 us with 4).
-// Examples (us, 8 strips and one tile -> chosen): 4096 x 4096 M = 16 15.0 -> 10.3; 1024 x 4096 M = 64 14.6 -> 9.8;
-// 14336 x 4096 M = 48 41 -> 32, M = 128 65 -> 53, M = 512 234 -> 201; 4096 x 4096 M = 32 with two tiles would be 22.4
-// against 13.
+// operands are built once for both; the Q6_K kernel has no registers left for it), 4 strips and one tile, 12 strips and
+// one tile (Q4_K), each with the number of parts of K that estimates fastest.  Times in microseconds fitted to
+// measurements on MI355X (Q4_K, 1024 x 4096 .. 32000 x 4096 and 4096 x 14336, 2 .. 512 tokens; they hold within about
+// 15 %): 5 to the first super-block and for the stores (3.5 with 4 strips); a super-block takes a workgroup 2.0 (8 strips),
+// 3.2 (8 strips, two tiles), 1.5 (4 strips) or 2.6 (12 strips; 2.4 alone on its CU, but with every CU busy the memory
+// system gives the larger workgroups no more than the smaller), and no cut streams the weights faster than about
+// 5 TB/s; with K in parts 2.5 for publishing a part, plus the time in which the workgroup that arrives last reads every
+// part of its rows through one CU, at about 40 GB/s - with 16 parts of 8 strips that read alone took 6.5 us of 15
+// (4096 x 4096, M = 16: 15.0 us with 8 strips, 10.3 us with 4).
+// Examples (us, 8 strips, one tile and as many parts as fill the CUs -> chosen): 4096 x 4096 M = 16 15.0 -> 10.3;
+// 1024 x 4096 M = 64 14.6 -> 9.8; 14336 x 4096 M = 48 41 -> 32, M = 128 65 -> 53, M = 512 234 -> 201; 4096 x 4096 M = 32 with
+// two tiles would be 22.4 against 13; 11008 x 4096 (43 groups of 8 strips: six parts of K make 258 workgroups, two more
+// than there are CUs) M = 4 19.5 -> 13.7 with four parts, M = 32 29.9 -> 18.7 with 12 strips (29 groups, eight parts).
 GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t k) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
-  auto cut_for = [&](uint32_t waves, uint32_t nt) {
+  const double weight_us = double(n) * nsb * kSbBytes[f] / 5.0e6;      // the weights once at 5 TB/s: no cut is faster
+  auto cut_with = [&](uint32_t waves, uint32_t nt, uint32_t kparts) {
     GemmCut c{waves, nt, (n + 32u * waves - 1u) / (32u * waves), (tiles + nt - 1u) / nt, 1u, nsb, 0.0};
     const uint64_t units = uint64_t(c.groups) * c.tgroups;
-    c.kparts = g_tune_gemm_ksplit > 0 ? uint32_t(g_tune_gemm_ksplit) : uint32_t((uint64_t(d.cu_count) + units / 2u) / units);
-    c.kparts = std::min(std::max(c.kparts, 1u), nsb);
+    c.kparts = std::min(std::max(kparts, 1u), nsb);
     c.ksb = (nsb + c.kparts - 1u) / c.kparts;
     c.kparts = (nsb + c.ksb - 1u) / c.ksb;
     const uint64_t rounds = (units * c.kparts + uint64_t(d.cu_count) - 1u) / uint64_t(d.cu_count);
-    const double step = waves == 4u ? 1.5 : nt == 2u ? 3.2 : 2.0;
+    const double step = waves == 4u ? 1.5 : waves == 12u ? 2.6 : nt == 2u ? 3.2 : 2.0;
     const double last_kb = double(c.kparts) * waves * nt * (m > 8u ? 2.0 : 1.0);
-    c.us = (waves == 4u ? 3.5 : 5.0) + double(rounds) * c.ksb * step + (c.kparts > 1u ? 2.5 + last_kb / 40.0 : 0.0);
+    c.us = (waves == 4u ? 3.5 : 5.0) + std::max(double(rounds) * c.ksb * step, weight_us) +
+           (c.kparts > 1u ? 2.5 + last_kb / 40.0 : 0.0);
     return c;
   };
+  // the parts of K: as many as bring the workgroups to about the number of CUs, or fewer where that estimates faster (one
+  // workgroup more than there are CUs costs a whole second round)
+  auto cut_for = [&](uint32_t waves, uint32_t nt) {
+    const uint64_t units = uint64_t((n + 32u * waves - 1u) / (32u * waves)) * ((tiles + nt - 1u) / nt);
+    if (g_tune_gemm_ksplit > 0) return cut_with(waves, nt, uint32_t(g_tune_gemm_ksplit));
+    const uint32_t most = uint32_t(std::min<uint64_t>((uint64_t(d.cu_count) + units / 2u) / units, nsb));
+    GemmCut best = cut_with(waves, nt, most);
+    for (uint32_t kp = most; kp-- > 1u;) {
+      const GemmCut c = cut_with(waves, nt, kp);
+      if (c.us < best.us) best = c;
+    }
+    return best;
+  };
   const int tw = g_tune_gemm_waves, tt = g_tune_gemm_tiles;
-  GemmCut best = cut_for(tw == 4 ? 4u : 8u, 1u);
+  const bool twelve_ok = f == Q4K;      // (the other formats' weight tiles do not fit twelve times two into LDS)
+  GemmCut best = cut_for(tw == 4 ? 4u : tw == 12 && twelve_ok ? 12u : 8u, 1u);
   if (tw == 0 && tt != 2) {
     const GemmCut four = cut_for(4u, 1u);
     if (four.us < best.us) best = four;
+    if (twelve_ok) {
+      const GemmCut twelve = cut_for(12u, 1u);
+      if (twelve.us < best.us) best = twelve;
+    }
   }
-  if (tw != 4 && f != Q6K && tiles >= 2u && tt != 1) {
+  if (tw != 4 && tw != 12 && f != Q6K && tiles >= 2u && tt != 1) {
     const GemmCut two = cut_for(8u, 2u);
     if (tt == 2 || two.us < best.us) best = two;
   }
@@ -449,7 +474,7 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   uint32_t nsb_arg = nsb;
   uint64_t geom = uint64_t(ksb) | uint64_t(kparts) << 16 | uint64_t(groups) << 32 | uint64_t(tiles) << 48;
   void* margs[] = {&a, &w, &c, &cnt, &m, &n, &nsb_arg, &geom};
-  hipFunction_t fn = nt == 2u ? d->gemm_f16_t2[f] : d->gemm_f16[f][waves == 8u];
+  hipFunction_t fn = nt == 2u ? d->gemm_f16_t2[f] : waves == 12u ? d->gemm_f16_w12 : d->gemm_f16[f][waves == 8u];
   return hipModuleLaunchKernel(fn, uint32_t(padded * tgroups), 1, 1, 64 * waves, 1, 1, lds, stream, margs, nullptr);
 }
 
