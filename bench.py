@@ -321,7 +321,7 @@ def main() -> int:
             for b in bufs:
                 b.free()
 
-        # the GEMM entry points outside BASELINE's configurations: Q5_K / Q6_K and the legacy 18-byte format of
+        # the GEMM entry points outside the benchmark's named configurations: Q5_K / Q6_K and the legacy 18-byte format of
         # q4k_gemm_fused, 4096 x 4096
         n = k = 4096
         for fmt in ("q5k", "q6k"):
