@@ -146,11 +146,12 @@ TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
  * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels and bit-identical
  * results; but where trn_q4k_gemm keeps a per-stream scratch buffer that it allocates and grows on demand (partial
  * results of the parts of K and their arrival counters), this entry point uses a buffer that is part of the library
- * image: a static device array of 8 MiB + 64 KiB, of which every GPU the library runs on holds one copy until the
+ * image: a static device array of 16 MiB + 64 KiB, of which every GPU the library runs on holds one copy until the
  * process ends.  After the library's first use on the device (any launcher, or trn_ctx_set_current, loads the kernels
  * and looks the buffer's address up once) it calls nothing that allocates or frees.  A product that needs more
- * scratch than that returns TRN_ERROR_SCRATCH_TOO_SMALL and launches nothing (every shape up to 1.5 x the CU count
- * of 16-token x 256-row tiles fits; m = 1 and unaligned operands take kernels that need no scratch).  All calls on
+ * scratch than that returns TRN_ERROR_SCRATCH_TOO_SMALL and launches nothing (every cut of a product that the library
+ * chooses by itself needs at most 11.2 MB on 256 CUs; a cut forced with trn_set_tuning may need more, and the library then
+ * takes one that fits if there is one; m = 1 and unaligned operands take kernels that need no scratch).  All calls on
  * one GPU share that GPU's buffer: calls that overlap in time on different streams of one GPU race - keep them on
  * one stream, or order the streams.  The kernels leave the counters at zero for the next call. */
 TRN_API trn_status trn_q4k_gemm_noalloc(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);

@@ -11,7 +11,7 @@
 
 namespace {
 constexpr size_t kCounterBytes = size_t(1) << 16;                    // arrival counters at the front (kGemmCounterBytes)
-constexpr size_t kScratchBytes = kCounterBytes + (size_t(8) << 20);   // + partial results of the parts of K
+constexpr size_t kScratchBytes = kCounterBytes + (size_t(16) << 20);   // + partial results of the parts of K
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {};
 }  // namespace

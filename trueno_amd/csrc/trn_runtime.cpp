@@ -393,7 +393,14 @@ struct GemmCut { uint32_t waves, nt, groups, tgroups, kparts, ksb; double us; };
 // 1024 x 4096 M = 64 14.6 -> 9.8; 14336 x 4096 M = 48 41 -> 32, M = 128 65 -> 53, M = 512 234 -> 201; 4096 x 4096 M = 32 with
 // two tiles would be 22.4 against 13; 11008 x 4096 (43 groups of 8 strips: six parts of K make 258 workgroups, two more
 // than there are CUs) M = 4 19.5 -> 13.7 with four parts, M = 32 29.9 -> 18.7 with 12 strips (29 groups, eight parts).
-GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t k) {
+// part_cap: the most bytes of partial sums the caller has room for; cuts that need more are left out (us = kCutDoesNotFit
+// when none fits).
+constexpr double kCutDoesNotFit = 1e30;
+size_t gemm_part_bytes(uint32_t kparts, uint32_t tiles, uint32_t groups, uint32_t waves) {
+  // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
+  return kparts > 1u ? (size_t(kparts) * tiles * groups * waves * 2048u + 255u) & ~size_t(255) : 0u;
+}
+GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t k, size_t part_cap = ~size_t(0)) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
   const double weight_us = double(n) * nsb * kSbBytes[f] / 5.0e6;      // the weights once at 5 TB/s: no cut is faster
   auto cut_with = [&](uint32_t waves, uint32_t nt, uint32_t kparts) {
@@ -407,6 +414,7 @@ GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t
     const double last_kb = double(c.kparts) * waves * nt * (m > 8u ? 2.0 : 1.0);
     c.us = (waves == 4u ? 3.5 : 5.0) + std::max(double(rounds) * c.ksb * step, weight_us) +
            (c.kparts > 1u ? 2.5 + last_kb / 40.0 : 0.0);
+    if (gemm_part_bytes(c.kparts, tiles, c.groups, waves) > part_cap) c.us = kCutDoesNotFit;
     return c;
   };
   // the parts of K: as many as bring the workgroups to about the number of CUs, or fewer where that estimates faster (one
@@ -448,15 +456,15 @@ hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint6
   const uint32_t kGemmWTileBytes = 32u * kSbBytes[f];
   // Q6_K: one weight tile per wave, rows 240 bytes apart (q6k_lds_bytes of the kernel's header)
   const uint32_t kGemmQ6TileBytes = 32u * 240u;
-  const GemmCut cut = gemm_cut(*d, f, m, n, k);
+  // a caller's own scratch buffer: only cuts whose partial sums fit behind the counters
+  const size_t part_cap = ext_base == 0 ? ~size_t(0) : ext_cap > kGemmCounterBytes ? ext_cap - kGemmCounterBytes : 0u;
+  const GemmCut cut = gemm_cut(*d, f, m, n, k, part_cap);
   const uint32_t waves = cut.waves, nt = cut.nt, groups = cut.groups, tgroups = cut.tgroups, kparts = cut.kparts, ksb = cut.ksb;
   const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
                                 : 2u * nt * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
-  auto up = [](size_t v) { return (v + 255u) & ~size_t(255); };
   // with several parts of K: one arrival counter per (group of strips, token tile)
   const size_t cnt_bytes = kparts > 1u ? size_t(groups) * tgroups * 4u : 0u;
-  // per part of K, token tile and strip of 32 rows: 64 lanes x 8 sums
-  const size_t part_bytes = kparts > 1u ? up(size_t(kparts) * tiles * groups * waves * 2048u) : 0u;
+  const size_t part_bytes = gemm_part_bytes(kparts, tiles, groups, waves);
   // the counters sit at the front of a region that only grows, so a larger product finds zeros there too (the
   // kernel puts every counter it used back to zero)
   const size_t cnt_cap = kGemmCounterBytes, need = cnt_cap + part_bytes;
