@@ -383,7 +383,7 @@ struct GemmCut { uint32_t waves, nt, groups, tgroups, kparts, ksb; double us; };
 // operands are built once for both; the Q6_K kernel has no registers left for it), 4 strips and one tile, 12 strips and
 // one tile (Q4_K), each with the number of parts of K that estimates fastest.  Times in microseconds fitted to
 // measurements on MI355X (Q4_K, 1024 x 4096 .. 32000 x 4096 and 4096 x 14336, 2 .. 512 tokens; they hold within about
-// 15 %): 5 to the first super-block and for the stores (3.5 with 4 strips); a super-block takes a workgroup 2.0 (8 strips),
+// 15 %): 4 to the first super-block and for the stores (3.5 with 4 strips); a super-block takes a workgroup 2.0 (8 strips),
 // 3.2 (8 strips, two tiles), 1.5 (4 strips) or 2.6 (12 strips; 2.4 alone on its CU, but with every CU busy the memory
 // system gives the larger workgroups no more than the smaller), and no cut streams the weights faster than about
 // 5 TB/s; with K in parts 2.5 for publishing a part, plus the time in which the workgroup that arrives last reads every
@@ -412,7 +412,7 @@ GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t
     const uint64_t rounds = (units * c.kparts + uint64_t(d.cu_count) - 1u) / uint64_t(d.cu_count);
     const double step = waves == 4u ? 1.5 : waves == 12u ? 2.6 : nt == 2u ? 3.2 : 2.0;
     const double last_kb = double(c.kparts) * waves * nt * (m > 8u ? 2.0 : 1.0);
-    c.us = (waves == 4u ? 3.5 : 5.0) + std::max(double(rounds) * c.ksb * step, weight_us) +
+    c.us = (waves == 4u ? 3.5 : 4.0) + std::max(double(rounds) * c.ksb * step, weight_us) +
            (c.kparts > 1u ? 2.5 + last_kb / 40.0 : 0.0);
     if (gemm_part_bytes(c.kparts, tiles, c.groups, waves) > part_cap) c.us = kCutDoesNotFit;
     return c;
