@@ -191,6 +191,26 @@ def test_gemm_ffn_shape_w_11008x4096(gpu, fmt, m):
     assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
 
 
+def _random_shapes():
+    rng = np.random.default_rng(20251125)
+    for i in range(15):
+        fmt = MFMA_FORMATS[i % 3]
+        k = 256 * int(rng.integers(1, 33))
+        n = int(rng.integers(1, 5000)) if i % 3 else 32 * int(rng.integers(1, 150))
+        m = int(rng.choice([2, 3, 5, 9, 16, 17, 31, 33, 48, 64, 65, 100, 130, 257]))
+        yield fmt, m, n, k, i
+
+
+@pytest.mark.parametrize("fmt,m,n,k,i", list(_random_shapes()))
+def test_gemm_random_shapes(gpu, fmt, m, n, k, i):
+    """Shapes drawn at random (fixed seed): whatever cut of the product the library's estimate picks for them - strips per
+    workgroup, token tiles per workgroup, parts of K of unequal length - the result is within tolerance."""
+    buf, a = kq.gen_matrix(fmt, 1000 + i, n, k), kq.gen_x(2000 + i, m, k)
+    c = gpu_gemm(gpu, fmt, buf, a, m, n, k)
+    assert np.all(np.isfinite(c))
+    assert kq.rel_l2(c, _c64(fmt, buf, a, n, k)) <= TOL
+
+
 @pytest.mark.parametrize("fmt", MFMA_FORMATS)
 def test_gemm_parts_of_k(gpu, fmt):
     """However K is cut into parts the result stays within tolerance, and the same cut gives the same bits on
