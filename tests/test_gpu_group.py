@@ -57,6 +57,41 @@ CASES = {
 }
 
 
+def _random_list(seed, entries=28):
+    """A list whose entries read buffers that earlier entries wrote (or x) and write new or existing buffers: read-after-
+    write, write-after-read and write-after-write dependencies at random, three formats, ragged row counts."""
+    rng = np.random.default_rng(seed)
+    sizes = {"x": 256 * int(rng.integers(1, 20))}
+    written, specs = ["x"], []
+    for i in range(entries):
+        src = written[int(rng.integers(0, len(written)))]
+        k = sizes[src] // 256 * 256
+        if k == 0:
+            src, k = "x", sizes["x"]
+        dst = f"b{i}"
+        if rng.random() < 0.35:
+            cands = [b for b in sizes if b != src and b != "x"]
+            if cands:
+                dst = cands[int(rng.integers(0, len(cands)))]
+        if dst not in sizes:
+            sizes[dst] = int(rng.choice([37, 256, 300, 512, 1024, 1500, 2816, 4352, 5000]))
+        specs.append((("q4k", "q5k", "q6k")[int(rng.integers(0, 3))], sizes[dst], k, src, dst, int(rng.integers(0, 2))))
+        if dst not in written:
+            written.append(dst)
+    return specs, sizes["x"]
+
+
+@pytest.mark.parametrize("seed", range(100, 105))
+def test_random_lists_grouped_equal_separate(gpu, seed):
+    specs, x_len = _random_list(seed)
+    plan = []
+    sep, _ = _run(gpu, specs, x_len, 1)
+    got, _ = _run(gpu, specs, x_len, 0, plan)
+    assert max(plan) + 1 < len(specs)          # something was grouped
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), (seed, name)
+
+
 @pytest.mark.parametrize("case", sorted(CASES))
 def test_grouped_equals_separate(gpu, case):
     specs, x_len = CASES[case]
