@@ -17,8 +17,8 @@ GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,
 h <- down) are timed too: `strict_decoder_chain` in `config`.
 
 Prints one JSON line.  `roofline`: the dominant kernel (kq_gemv_group: the launches that carry several
-independent entries, 28 per pass, 3.99 of the 4.13 GB), its launches of one pass timed with HIP events on
-their stream, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
+independent entries, 15 per pass, 4.02 of the 4.13 GB), those launches timed with HIP events on their stream
+over as many rounds as the headline has passes, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other
 benchmark configurations, timed as launches back to back over at least 1 GiB of distinct copies
 (200 launches, median of 5 batches), one copy over and over ("hot": from the last-level cache), and
@@ -179,17 +179,21 @@ def main() -> int:
             groups.append(g)
             grp_bytes += sum(entry_bytes[i] for i in members[l])
     n_grp = len(groups)
+    # as many rounds of these launches between the two events as the headline has passes (the clocks of a memory-bound
+    # run wander by several percent over milliseconds: one round alone read 55-66 us per launch on one box), three such
+    # measurements, the median
     grp_ms = []
-    for _ in range(5):
+    for _ in range(3):
         for g in groups:
             g.launch(stream)
         stream.synchronize()
         L.trn_event_record(e0, stream.raw())
-        for g in groups:
-            g.launch(stream)
+        for _ in range(args.steps):
+            for g in groups:
+                g.launch(stream)
         L.trn_event_record(e1, stream.raw())
         stream.synchronize()
-        grp_ms.append(elapsed_ms(e0, e1) / n_grp)
+        grp_ms.append(elapsed_ms(e0, e1) / (n_grp * args.steps))
     grp_ms = sorted(grp_ms)[len(grp_ms) // 2]
     grp_bytes_per_launch = grp_bytes / n_grp
     achieved = grp_bytes_per_launch / (grp_ms * 1e-3) / 1e9

@@ -98,6 +98,7 @@ std::atomic<int> g_tune_gemm_tiles{0};      // token tiles per workgroup of the 
 std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 std::atomic<int> g_tune_attention_min_steps{0};
 std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped launch may look ahead over (0: 16)
+std::atomic<int> g_tune_group_waves{0};        // least waves per workgroup of a grouped launch (0: what the widest entry needs)
 std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8; at most 16)
 std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
@@ -644,11 +645,12 @@ uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u +
 // of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
 // barrier between phases.  *handled = false (and hipSuccess): not possible here, issue the list the plain way.
 constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (kGroupEntries of the kernel)
-// Entries a launch takes by default.  More is not better: on the 7B pass with activation buffers per layer, launches of
-// 8 entries (138 MB, 30 launches) take 880 us, of 12 entries 940 us, of 16 entries (275 MB, 16 launches) 1075-1095 us - with
-// more entries each one's share of the workgroups gets coarse (9 of 256 for a 4096 x 4096 matrix beside a 4096 x 11008
-// one) and the launch ends as unevenly.
-constexpr uint32_t kGroupDefault = 8;
+// Entries a launch takes by default: as many as the kernel holds, looked for among the next 32 of the list.  On the 7B
+// pass with activation buffers per layer: 8 entries (138 MB a launch, 30 launches) 879 us, 12 of the next 24 (21
+// launches) 820 us, 14 of 28 (18) 821 us, 16 of 32 (16 launches of 270 MB) 823 us; the launches of 12-16 entries run at
+// 4.8-5.4 TB/s against 4.3-4.7 for 8.  (Before the workgroups of a launch were kept within the number resident at once -
+// launch_gemv_group - sixteen entries measured 1075 us: shares rounded up to 260 workgroups for 256 places.)
+constexpr uint32_t kGroupDefault = 16;
 bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
   return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
          gemv_geometry(*dk, d.k, d.n).fits;
@@ -1298,6 +1300,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     if (!alone.fits) return hipErrorInvalidValue;
     waves = std::max(waves, alone.block / 64u);
   }
+  if (g_tune_group_waves > 0) waves = std::max(waves, std::min(uint32_t(g_tune_group_waves), kGemvMaxWaves));
   // What an entry costs a workgroup is not only its bytes: with k > 4096 every workgroup stages a larger vector and
   // the waves that share a row meet in LDS.  Measured on [Q6_K 4096x11008 + 3 x Q4_K 4096x4096]: with shares by bytes
   // the wide entry's workgroups end 5 us after the others; counting its bytes 1.6-1.75 times is best (0.3 per
@@ -1314,27 +1317,54 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   GemvGroupHost g{};
   uint32_t first[kGroupMax + 1] = {};
   uint32_t lds = 0;
-  for (uint32_t i = 0; i < len; ++i) {
+  // rows per workgroup and workgroups of entry i when it is given `share` workgroups (0 rows: it does not fit the engine)
+  struct Cut { uint64_t rows; uint32_t grid; };
+  auto cut_of = [&](uint32_t i, uint64_t share) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves), groups = waves / sw;
-    const double bytes = cost_of(e);
-    const uint64_t share = std::max<uint64_t>(1, uint64_t(target * bytes / total_bytes + 0.5));
     const uint64_t x_bytes = uint64_t(e.k) * 4u;
-    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags, 0u, 0u};
-    g.cold[i] = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
     // workgroups of 8 waves or more hand their row batches out among the waves: a share need not be a whole
     // number of rounds of all waves
     const uint32_t ug = waves >= 8u ? kGemvRowsPerBatch : kGemvRowsPerBatch * groups;
     uint64_t rows = (uint64_t(e.n) + share - 1) / share;
     rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
-    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return hipErrorInvalidValue;
+    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return Cut{0u, 0u};
     const uint64_t max_rows = (kFastLdsLimit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
     rows = std::min<uint64_t>(rows, max_rows);
-    const uint32_t grid = uint32_t((uint64_t(e.n) + rows - 1) / rows);
-    lds = std::max<uint32_t>(lds, uint32_t(x_bytes + uint64_t(sw) * rows * 4u + kLdsScratch));
-    first[i + 1] = first[i] + grid;
+    return Cut{rows, uint32_t((uint64_t(e.n) + rows - 1) / rows)};
+  };
+  uint64_t share[kGroupMax] = {};
+  Cut cut[kGroupMax] = {};
+  uint64_t total_grid = 0;
+  for (uint32_t i = 0; i < len; ++i) {
+    share[i] = std::max<uint64_t>(1, uint64_t(target * cost_of(descs[i]) / total_bytes + 0.5));
+    cut[i] = cut_of(i, share[i]);
+    if (cut[i].rows == 0) return hipErrorInvalidValue;
+    total_grid += cut[i].grid;
+  }
+  // Rounded shares can add up to a few workgroups more than are resident at once, and a workgroup that has to wait for
+  // a place runs when the others are done: the launch takes twice as long (measured: 66 us instead of 44 for twelve
+  // entries in 260 workgroups of 12 waves on 256 CUs).  Take workgroups from the entries that have the most until
+  // all fit.
+  for (uint32_t guard = 0; total_grid > uint64_t(target) && guard < 4096u; ++guard) {
+    uint32_t big = 0;
+    for (uint32_t i = 1; i < len; ++i)
+      if (cut[i].grid > cut[big].grid) big = i;
+    if (cut[big].grid <= 1u || share[big] <= 1u) break;
+    const uint32_t before = cut[big].grid;
+    do cut[big] = cut_of(big, --share[big]); while (share[big] > 1u && cut[big].grid >= before);
+    if (cut[big].grid >= before) break;            // (its rows per workgroup are at the limit of LDS)
+    total_grid -= before - cut[big].grid;
+  }
+  for (uint32_t i = 0; i < len; ++i) {
+    const trn_gemv_desc& e = descs[i];
+    const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves);
+    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags, 0u, 0u};
+    g.cold[i] = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
+    lds = std::max<uint32_t>(lds, uint32_t(uint64_t(e.k) * 4u + uint64_t(sw) * cut[i].rows * 4u + kLdsScratch));
+    first[i + 1] = first[i] + cut[i].grid;
     g.hot[i].first_block = first[i];
-    g.hot[i].num_blocks = grid;
+    g.hot[i].num_blocks = cut[i].grid;
   }
   for (uint32_t i = len; i < kGroupMax; ++i) first[i + 1] = first[len];   // entries that do not exist own no workgroup
   if (first[len] > 0xFFFFu) return hipErrorInvalidValue;                  // the table holds 16 bits per entry
@@ -1575,6 +1605,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemm_waves")) { g_tune_gemm_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_window")) { g_tune_group_window = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_max")) { g_tune_group_max = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_waves")) { g_tune_group_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "group_slab_weight")) { g_tune_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_per_cu")) { g_tune_attention_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_min_steps")) { g_tune_attention_min_steps = value; return TRN_SUCCESS; }
