@@ -17,7 +17,7 @@ GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,
 h <- down) are timed too: `strict_decoder_chain` in `config`.
 
 Prints one JSON line.  `roofline`: the dominant kernel (kq_gemv_group: the launches that carry several
-independent entries, 15 per pass, 4.02 of the 4.13 GB), those launches timed with HIP events on their stream
+independent entries and the head alone: the 16 launches of a pass), those launches timed with HIP events on their stream
 over as many rounds as the headline has passes, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
 (oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other
 benchmark configurations, timed as launches back to back over at least 1 GiB of distinct copies
@@ -159,9 +159,9 @@ def main() -> int:
 
     # ---- dominant kernel: kq_gemv_group.  The library puts entries that are independent of one another (and of what
     #      they would overtake) into one launch of this kernel; trn_kquant_gemv_plan says which entry of the pass goes
-    #      into which launch.  The launches of the pass that hold two or more entries (all of it but the head, which
-    #      takes the single-GEMV kernel) are issued here one list each, in pass order, back to back on the stream,
-    #      bracketed by HIP events on that stream.
+    #      into which launch.  A launch of two or more entries runs this kernel, and so does a single matrix of 64 MB or
+    #      more (the head): on this pass that is every launch.  They are issued here one list each, in pass order, back
+    #      to back on the stream, bracketed by HIP events on that stream.
     launch_of = batch.plan()
     members = {}
     for i, l in enumerate(launch_of):
@@ -173,7 +173,7 @@ def main() -> int:
     print("[bench] launches of the pass: " + ", ".join(f"{c} x {sig}" for sig, c in kinds.items()), file=sys.stderr, flush=True)
     groups, grp_bytes = [], 0
     for l in sorted(members):
-        if len(members[l]) >= 2:
+        if len(members[l]) >= 2 or entry_bytes[members[l][0]] >= 64e6 + 4 * (32000 + 4096):
             g = batch.subset(members[l])
             assert len(set(g.plan())) == 1, "a launch of the pass, issued alone, must again be one launch"
             groups.append(g)

@@ -292,7 +292,7 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * "group_off": 1 = in mode 0 one launch per entry; "group_max": most entries in a launch (0 = 16, the most the kernel holds); "group_window":
  * how far down the list a launch looks for entries (0 = 32); "group_waves": least waves per workgroup of such a launch (0 = what
  * its widest entry needs); "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch
- * shares out its workgroups (0 = 30).
+ * shares out its workgroups (0 = 40).
  * "gemm_mfma_off": 1 = the k-quant GEMMs never take the matrix-core form; "gemm_k_parts": into how many parts
  * that form cuts K; "gemm_waves": 4, 8 or (Q4_K) 12 strips of 32 rows per workgroup; "gemm_tiles": 1 or 2 tiles of 16 tokens per
  * workgroup (0 for each of the three = chosen from the shape by an estimated time; any of them set also keeps a

@@ -1300,14 +1300,19 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     if (!alone.fits) return hipErrorInvalidValue;
     waves = std::max(waves, alone.block / 64u);
   }
-  if (g_tune_group_waves > 0) waves = std::max(waves, std::min(uint32_t(g_tune_group_waves), kGemvMaxWaves));
+  // At least 8 waves to a workgroup (they hand their row batches out among themselves, and a CU stages a vector once or
+  // twice instead of three times): sixteen one-slab entries of 247 MB in one launch 55.4 us with 4 waves, 51.4 with 8,
+  // 50.9 with 12; the 7B pass with shared activation buffers (65 launches of three or four entries) 1070 -> 1062 us,
+  // with 12 waves 1076 us.
+  waves = std::max(waves, g_tune_group_waves > 0 ? std::min(uint32_t(g_tune_group_waves), kGemvMaxWaves) : 8u);
   // What an entry costs a workgroup is not only its bytes: with k > 4096 every workgroup stages a larger vector and
   // the waves that share a row meet in LDS.  Measured on [Q6_K 4096x11008 + 3 x Q4_K 4096x4096]: with shares by bytes
-  // the wide entry's workgroups end 5 us after the others; counting its bytes 1.6-1.75 times is best (0.3 per
-  // further slab of 4096 columns; "group_slab_weight" overrides the percentage).
+  // the wide entry's workgroups end 5 us after the others; counting its bytes 1.6-1.8 times is best (0.4 per
+  // further slab of 4096 columns; "group_slab_weight" overrides the percentage.  The 7B pass in launches of sixteen
+  // entries: 932 / 875 / 832 / 800 / 794 / 803 / 880 us with 1 / 10 / 20 / 30 / 40 / 50 / 70 percent).
   auto cost_of = [&](const trn_gemv_desc& e) {
     const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
-    const double per_slab = (g_tune_slab_weight > 0 ? int(g_tune_slab_weight) : 30) / 100.0;
+    const double per_slab = (g_tune_slab_weight > 0 ? int(g_tune_slab_weight) : 40) / 100.0;
     return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
   };
   for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
@@ -1355,6 +1360,26 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     do cut[big] = cut_of(big, --share[big]); while (share[big] > 1u && cut[big].grid >= before);
     if (cut[big].grid >= before) break;            // (its rows per workgroup are at the limit of LDS)
     total_grid -= before - cut[big].grid;
+  }
+  // ... and where places are left over, give them to the entries whose workgroups have the most to do
+  for (uint32_t guard = 0; total_grid < uint64_t(target) && guard < 4096u; ++guard) {
+    int best = -1;
+    double most = 0.0;
+    Cut best_cut{};
+    uint64_t best_share = 0;
+    for (uint32_t i = 0; i < len; ++i) {
+      const double per_wg = cost_of(descs[i]) / double(descs[i].n) * double(cut[i].rows);
+      if (per_wg <= most) continue;
+      uint64_t sh = share[i];
+      Cut c = cut[i];
+      while (c.grid <= cut[i].grid && sh < share[i] + 64u) c = cut_of(i, ++sh);       // the next share that changes the cut
+      if (c.grid <= cut[i].grid || total_grid - cut[i].grid + c.grid > uint64_t(target)) continue;
+      best = int(i); most = per_wg; best_cut = c; best_share = sh;
+    }
+    if (best < 0) break;
+    total_grid += best_cut.grid - cut[best].grid;
+    cut[best] = best_cut;
+    share[best] = best_share;
   }
   for (uint32_t i = 0; i < len; ++i) {
     const trn_gemv_desc& e = descs[i];
@@ -1463,7 +1488,10 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   std::vector<trn_gemv_desc> group;
   for (const std::vector<uint32_t>& members : launches) {
     const trn_gemv_desc& head = descs[members[0]];
-    if (members.size() >= 2 || (desc_extended(head) && list_groupable(dk, head))) {
+    // a large matrix alone (the 108 MB head of the 7B pass) is 2-4 us faster as a group of one: workgroups of 8 waves that
+    // hand their rows out among themselves; smaller ones alone (37 MB, 9 MB) are slower that way
+    const bool big_single = list_groupable(dk, head) && double(head.n) * (head.k / 256u) * kSbBytes[head.fmt - 4] >= 64e6;
+    if (members.size() >= 2 || big_single || (desc_extended(head) && list_groupable(dk, head))) {
       group.clear();
       for (uint32_t m : members) group.push_back(descs[m]);
       e = launch_gemv_group(dk, stream, group.data(), uint32_t(group.size()));
