@@ -645,6 +645,8 @@ uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u +
 // of 12 waves per CU, per phase dealt to the phase's entries in proportion to their bytes, a device-wide
 // barrier between phases.  *handled = false (and hipSuccess): not possible here, issue the list the plain way.
 constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (kGroupEntries of the kernel)
+// what a further slab of 4096 columns adds to the cost of an entry's bytes when workgroups are shared out (launch_gemv_group)
+constexpr double kSlabCost = 0.4;
 // Entries a launch takes by default: as many as the kernel holds, looked for among the next 32 of the list.  On the 7B
 // pass with activation buffers per layer: 8 entries (138 MB a launch, 30 launches) 879 us, 12 of the next 24 (21
 // launches) 820 us, 14 of 28 (18) 821 us, 16 of 32 (16 launches of 270 MB) 823 us; the launches of 12-16 entries run at
@@ -714,7 +716,7 @@ hipError_t launch_phases(DeviceKernels* d, ChainWorkspace* ws, hipStream_t strea
       // cost, not bytes: a Q6_K byte takes longer than a Q4_K byte (measured: the workgroups of a Q6_K entry with
       // a byte share ended 5 us after those of its Q4_K neighbours)
       const uint32_t slabs_i = std::min((descs[a + i].k / 256u + 15u) / 16u, kWaves);
-      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4] * (1.0 + 0.3 * (slabs_i - 1u));
+      bytes[i] = double(descs[a + i].n) * (descs[a + i].k / 256u) * kSbBytes[descs[a + i].fmt - 4] * (1.0 + kSlabCost * (slabs_i - 1u));
       total += bytes[i];
     }
     // shares: at least one workgroup each, the rest in proportion to the bytes (largest remainders first)
@@ -1312,7 +1314,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   // entries: 932 / 875 / 832 / 800 / 794 / 803 / 880 us with 1 / 10 / 20 / 30 / 40 / 50 / 70 percent).
   auto cost_of = [&](const trn_gemv_desc& e) {
     const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
-    const double per_slab = (g_tune_slab_weight > 0 ? int(g_tune_slab_weight) : 40) / 100.0;
+    const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
     return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
   };
   for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
