@@ -1374,7 +1374,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
       if (per_wg <= most) continue;
       uint64_t sh = share[i];
       Cut c = cut[i];
-      while (c.grid <= cut[i].grid && sh < share[i] + 64u) c = cut_of(i, ++sh);       // the next share that changes the cut
+      while (c.grid <= cut[i].grid && sh < share[i] + 16u) c = cut_of(i, ++sh);       // the next share that changes the cut
       if (c.grid <= cut[i].grid || total_grid - cut[i].grid + c.grid > uint64_t(target)) continue;
       best = int(i); most = per_wg; best_cut = c; best_share = sh;
     }
