@@ -1,6 +1,9 @@
 """Shared helpers for the GPU parity tests: upload, launch through the C ABI, download."""
 from __future__ import annotations
 
+import json
+import os
+
 import numpy as np
 
 import trueno_amd as t
@@ -9,6 +12,21 @@ from trueno_amd import kernels as K
 GEMV_KERNEL = {"q4k": t.Q4KGemvKernel, "q5k": t.Q5KGemvKernel, "q6k": t.Q6KGemvKernel}
 GEMM_KERNEL = {"q4k": t.QuantizeKernel.ggml, "q5k": t.Q5KKernel, "q6k": t.Q6KKernel}
 SB = {"q4k": 144, "q5k": 176, "q6k": 210}
+
+# Our error against fp64 may be at most this multiple of the error of an f32 evaluation in the reference's own
+# summation order (trueno-gpu/src/kernels/quantize.rs:1412, 1482-1518).  The clause is "no worse than": 1.0, plus a
+# sampling margin - both errors are sums over a few thousand rounding errors, so their ratio scatters by about
+# 1 / sqrt(rows) around its expectation (1.6 % with 4096 rows, 2.2 % with 2048, 3.1 % with 1024).
+REF_SLACK = 1.05
+RATIO_LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "ref_order_ratios.jsonl")
+
+
+def record_ratio(kind: str, fmt: str, m: int, n: int, k: int, rows: int, ours: float, ref: float) -> None:
+    """one line per measured shape: our relative L2 error against fp64 over the reference-order f32 evaluation's"""
+    os.makedirs(os.path.dirname(RATIO_LOG), exist_ok=True)
+    with open(RATIO_LOG, "a") as f:
+        f.write(json.dumps({"kind": kind, "fmt": fmt, "m": m, "n": n, "k": k, "rows": rows, "ours": ours, "reference_order": ref,
+                            "ratio": ours / ref if ref > 0 else None}) + "\n")
 
 
 def gpu_dequant(gpu, fmt: str, buf: np.ndarray, policy: int = 0, w_offset: int = 0) -> np.ndarray:

@@ -474,6 +474,77 @@ def test_reference_order_emulation(fmt, co):
     assert 0 < kq.rel_l2(a, kq.gemv_fp64(w, x)) < 1e-6
 
 
+def _q6k_all_ones(n_sb):
+    """Q6_K super-blocks whose 256 weights are all 1.0: d = 1 (f16 0x3C00), every scale 1, every quant 33
+    (low nibble 1 in ql, two-bit field 2 in qh), so w = d * sc * (q - 32) = 1."""
+    b = np.zeros((n_sb, 210), np.uint8)
+    b[:, :128] = 0x11
+    b[:, 128:192] = 0xAA
+    b[:, 192:208] = 1
+    b[:, 208:210] = [0x00, 0x3C]
+    return b.reshape(-1)
+
+
+def _sum_in_order(x, owner, chain, tree):
+    """f32 sum of x (one super-block, all weights 1) for a lane ownership, a chain direction and a tree: a
+    deliberately general helper, used only to show that OTHER orders miss the hand-worked values below."""
+    f = np.float32
+    acc = []
+    for t in range(32):
+        p = f(0)
+        for j in chain:
+            p = f(p + f(x[owner(t, j)]))
+        acc.append(p)
+    for step in tree:
+        # steps falling from 16: the shuffle-down tree (lane t takes lane t + step); rising from 1: neighbours first
+        for t in (range(step) if tree[0] == 16 else range(0, 32, 2 * step)):
+            acc[t] = f(acc[t] + acc[t + step])
+    return float(acc[0])
+
+
+def test_reference_order_hand_worked(co):
+    """The yardstick of "no worse than the reference's own f32 result", pinned by cases worked by hand from
+    quantize.rs:1412, 1482-1518 (lane t of 32 owns values t + 32 j; p = 0, p = fma(x, w, p) for j = 0..7;
+    acc += p per super-block; then acc[i] += acc[i + 16], + 8, + 4, + 2, + 1; lane 0 is the result).
+
+    All weights are 1 and x holds a few powers of two; B = 2^24, where f32 has spacing 2 (B + 1 rounds to B,
+    1 - B is exact).  Values of x that are not zero, by index i = t + 32 j:
+        i = 0: 1    i = 32: B    i = 64: -B      lane 0:  (1 + B) - B = B - B = 0          (the 1 is lost)
+        i = 8: 1                                 lane 8:  1
+        i = 4: B    i = 20: 1    i = 12: -B      lanes 4, 20, 12: B, 1, -B
+        i = 2: 0.5  i = 1: 0.25                  lanes 2, 1
+    tree, step 16:  a0 = p0 + p16 = 0;  a8 = p8 + p24 = 1;  a4 = p4 + p20 = B + 1 = B (lost);  a12 = -B
+          step 8:   a0 = 0 + 1 = 1;  a4 = B - B = 0;  step 4: a0 = 1 + 0 = 1;  step 2: a0 = 1 + 0.5;  step 1: + 0.25
+    so y = 1.75, where the exact sum is 3.75.  Other orders give other numbers: a chain from j = 7 down keeps lane 0's
+    1 (2.75); a tree of neighbours first (1, 2, 4, 8, 16) gives 2; lanes owning 8 t .. 8 t + 7 give 5."""
+    B = np.float32(2.0 ** 24)
+    x = np.zeros(256, np.float32)
+    for i, v in ((0, 1), (32, B), (64, -B), (8, 1), (4, B), (20, 1), (12, -B), (2, 0.5), (1, 0.25)):
+        x[i] = v
+    assert float(x.astype(np.float64).sum()) == 3.75
+    w = np.ones((1, 256), np.float32)
+    assert kq.gemv_ref_order_fp32(w, x)[0] == np.float32(1.75)
+    blocks = _q6k_all_ones(1)
+    assert np.all(kq.dequant_matrix("q6k", blocks, 1, 256) == 1.0)
+    assert co.gemv_ref_order_f32("q6k", blocks, x, 256, 1)[0] == np.float32(1.75)
+    # the case tells the orders apart
+    strided, contiguous = (lambda t, j: t + 32 * j), (lambda t, j: 8 * t + j)
+    down_tree, up_tree = (16, 8, 4, 2, 1), (1, 2, 4, 8, 16)
+    assert _sum_in_order(x, strided, range(8), down_tree) == 1.75
+    assert _sum_in_order(x, strided, range(7, -1, -1), down_tree) == 2.75
+    assert _sum_in_order(x, strided, range(8), up_tree) == 2.0
+    assert _sum_in_order(x, contiguous, range(8), down_tree) == 5.0
+
+    # Two super-blocks: the partial sum of a super-block is formed on its own and then added (quantize.rs:1412, 1486).
+    # Lane 0: super-block 0 holds B; super-block 1 holds 1 (j = 0) and 1 (j = 1): p = 2, acc = B + 2 exactly.  Adding
+    # the values to acc one by one would lose both: B + 1 = B, B + 1 = B.
+    x2 = np.zeros(512, np.float32)
+    x2[0], x2[256], x2[256 + 32] = B, 1, 1
+    want = np.float32(2.0 ** 24 + 2)
+    assert kq.gemv_ref_order_fp32(np.ones((1, 512), np.float32), x2)[0] == want
+    assert co.gemv_ref_order_f32("q6k", _q6k_all_ones(2), x2, 512, 1)[0] == want
+
+
 def test_row_layout():
     """row n starts at byte n * (k/256) * SB (quantize.rs:1219-1224)"""
     n, k = 5, 768

@@ -45,7 +45,10 @@ struct ChainEntry {
   float eps;          // of the normalisation; 0 = kChainNormEps
   u32 pad;
 };
-enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u, CHAIN_SWIGLU_INPUT = 8u };
+enum : u32 { CHAIN_NORM_INPUT = 1u, CHAIN_BARRIER_BEFORE = 2u, CHAIN_SAME_X = 4u, CHAIN_SWIGLU_INPUT = 8u,
+             // set by the launcher, never by a caller: the rows of this (one-slab) entry are streamed through LDS
+             // (chain_step_stream); the launch's dynamic LDS then includes the waves' rings
+             CHAIN_STREAM_LDS = 16u };
 constexpr float kChainNormEps = 1e-6f;
 
 // silu(g) * u with the reference's instruction sequence (trueno-gpu/src/kernels/elementwise.rs:565-582)
@@ -112,6 +115,227 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
   return *s_flag != 0u;
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// The engine for matrices of at most 4096 columns (one slab: a wave covers whole rows), weights streamed through LDS.
+//
+// What the memory system gives a read depends on how it is asked.  Measured on MI355X, 258 MB per launch: the engine's
+// own pattern (every lane three 16-byte loads at its quarter of a 144-byte block, so each 128-byte line is asked for by
+// three instructions) reads 5.9-6.0 TB/s, and the same with non-temporal loads 4.5 TB/s (a line is fetched again by
+// every instruction that asks for a part of it); whole lines asked for once, by non-temporal loads of 1 KB contiguous
+// per wave instruction, arrive at 6.55-6.7 TB/s (1.4 GB per launch: 6.9 TB/s against 6.15 TB/s).  So here a batch of U
+// rows - U * row bytes, contiguous in memory - is copied to LDS as it lies (global_load_lds_dwordx4, non-temporal, no
+// registers held while it is on its way), two batches ahead per wave, and the lanes then read their quarter blocks
+// from LDS (Quarter::load_lds: the same pieces as Quarter::load takes from memory).  The arithmetic - and so every bit of
+// the result - is chain_step's.
+//
+// A batch may start at any even address (Q6_K rows of 210-byte blocks): the copy starts at the 16-byte boundary below it
+// and the reads are shifted by the difference.  Pieces beyond the end of the batch (or of the matrix) repeat its last
+// piece: every wave instruction is issued unconditionally, so the number of copies outstanding is known where the waits
+// are written (vmcnt counted by hand; all LDS traffic in asm, see kquant_quarter.hip.h).
+//   LDS: [k floats of x, swizzled][rows_per_block partial sums][64 group sums of squares][ring: waves * 2 * slot bytes]
+// ------------------------------------------------------------------------------------------------------------
+template <int FMT, int U> struct StreamSlot {
+  static constexpr u32 PIECES = (U * 16u * Quarter<FMT>::SB + 15u + 1023u) / 1024u;   // wave instructions per batch
+  static constexpr u32 BYTES = PIECES * 1024u;
+};
+
+__device__ __forceinline__ u32 lds_addr_of(const void* p) {
+  return static_cast<u32>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) uint8_t*)p));
+}
+__device__ __forceinline__ void dma16_nt(const uint8_t* src, u32 lds_addr) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)(uintptr_t)lds_addr, 16, 0, 2 /* nt */);
+}
+
+template <int FMT, int U>
+__device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* lds4, u32 block_id, u32 num_blocks, u32 block_threads) {
+  using Q = Quarter<FMT>;
+  using Slot = StreamSlot<FMT, U>;
+  constexpr u32 NL = Slot::PIECES;
+  const u32 tid = threadIdx.x, lane = tid & 63u, waves = block_threads >> 6;
+  const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(tid >> 6)));
+  const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;            // 1 <= nsb <= 16
+  u32 rows_per_block = (n_dim + num_blocks - 1) / num_blocks;
+  rows_per_block = ((rows_per_block + U - 1) / U) * U;
+  const u32 row0 = block_id * rows_per_block;
+  if (row0 >= n_dim) return true;                                  // the whole workgroup: nothing was touched yet
+  const u32 batches = rows_per_block / U;
+  const u32 sbl = lane >> 2, c = lane & 3u;
+  const u32 row_bytes = nsb * Q::SB;
+  const u32 batch_bytes = U * row_bytes;
+  const size_t total = static_cast<size_t>(n_dim) * row_bytes;
+
+  const u32 units = k_dim >> 2, xgroups = units >> 6;
+  const u32 lds_x = lds_addr_of(lds4);
+  const u32 lds_part = lds_x + 16u * units;
+  const u32 lds_ss = lds_part + 4u * rows_per_block;
+  const u32 lds_ring = ((lds_ss + 256u + 15u) & ~15u) + wave * (2u * Slot::BYTES);
+  __shared__ u32 s_next_stream;
+  const u32 lds_next = lds_addr_of(&s_next_stream);
+
+  // batch b of this workgroup into ring slot `slot`; returns the byte shift of the batch inside the slot
+  auto issue = [&](u32 b, u32 slot) -> u32 {
+    size_t off = static_cast<size_t>(row0 + b * U) * row_bytes;
+    if (off >= total) off = 0;                                       // a batch that does not exist: any valid bytes
+    const u32 avail = static_cast<u32>(total - off < batch_bytes ? total - off : batch_bytes);
+    const uint8_t* src = e.w + off;
+    const u32 shift = static_cast<u32>(reinterpret_cast<size_t>(src)) & 15u;
+    src -= shift;
+    const u32 last = (shift + avail - 1u) >> 4;                      // the last 16-byte piece that holds bytes of the batch
+    const u32 dst = lds_ring + slot * Slot::BYTES;
+#pragma unroll
+    for (u32 j = 0; j < NL; ++j) {
+      const u32 p = 64u * j + lane;
+      dma16_nt(src + 16u * (p < last ? p : last), dst + 1024u * j);
+    }
+    return shift;
+  };
+
+  // Activations first (loads return in order, and the vector is an L2 hit), then the first two batches of this wave,
+  // all unconditionally.  The loads of the vector are written in asm like the copies' waits: the compiler, which knows
+  // the copies only as memory operations that write LDS, would wait for all of them before it touches LDS at all.
+  constexpr u32 kXPre = 4;
+  const bool swiglu = (e.flags & CHAIN_SWIGLU_INPUT) != 0u;
+  u32x4 xv[kXPre], x2v[kXPre];
+#pragma unroll
+  for (u32 i = 0; i < kXPre; ++i) {
+    const u32 g = wave + i * waves;
+    const u32 unit = 64u * (g < xgroups ? g : 0u) + lane;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xv[i]) : "v"(reinterpret_cast<const f32x4*>(e.x) + unit) : "memory");
+  }
+  if (swiglu) {
+#pragma unroll
+    for (u32 i = 0; i < kXPre; ++i) {
+      const u32 g = wave + i * waves;
+      const u32 unit = 64u * (g < xgroups ? g : 0u) + lane;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(x2v[i]) : "v"(reinterpret_cast<const f32x4*>(e.x2) + unit) : "memory");
+    }
+  }
+  u32 cur = wave, nxt = wave + waves;
+  u32 shift_cur = issue(cur, 0u);
+  u32 shift_nxt = issue(nxt, 1u);
+  // the vector has landed when only the copies issued behind it are outstanding
+#pragma unroll
+  for (u32 i = 0; i < kXPre; ++i) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xv[i]) : "n"(2 * NL) : "memory");
+  if (swiglu) {
+#pragma unroll
+    for (u32 i = 0; i < kXPre; ++i) asm volatile("" : "+v"(x2v[i]));
+  }
+
+  const bool norm = (e.flags & CHAIN_NORM_INPUT) != 0u;
+  auto stage = [&](u32 g, f32x4 v) {
+    if (norm) {
+      const float sg = wave_sum(unit_sumsq(v));
+      if (lane == 0) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_ss + 4u * g), "v"(sg) : "memory");
+    }
+    if (e.gamma) {
+      const f32x4 gm = reinterpret_cast<const f32x4*>(e.gamma)[64u * g + lane];
+      v = f32x4{__fmul_rn(v.x, gm.x), __fmul_rn(v.y, gm.y), __fmul_rn(v.z, gm.z), __fmul_rn(v.w, gm.w)};
+    }
+    asm volatile("ds_write_b128 %0, %1" ::"v"(lds_x + 16u * Q::swz(64u * g + lane)), "v"(v) : "memory");
+  };
+  auto as_f32x4 = [](const u32x4& w) { return f32x4{__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w)}; };
+#pragma unroll
+  for (u32 i = 0; i < kXPre; ++i) {
+    const u32 g = wave + i * waves;
+    if (g < xgroups) {
+      f32x4 v = as_f32x4(xv[i]);
+      if (swiglu) {
+        const f32x4 g2 = as_f32x4(x2v[i]);
+        v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
+      }
+      stage(g, v);
+    }
+  }
+  for (u32 g = wave + kXPre * waves; g < xgroups; g += waves) {     // (workgroups of fewer than four waves)
+    f32x4 v = reinterpret_cast<const f32x4*>(e.x)[64u * g + lane];
+    if (swiglu) {
+      const f32x4 g2 = reinterpret_cast<const f32x4*>(e.x2)[64u * g + lane];
+      v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
+    }
+    stage(g, v);
+  }
+  if (tid == 0u) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_next), "v"(2u * waves) : "memory");
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+  {
+    const bool valid = sbl < nsb;
+    const u32 sbc = valid ? sbl : nsb - 1u;
+    float xr[64];
+    float sx[Q::NSUM];
+    {
+      u32x4 xq[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const u32 unit = (256u * sbc + Q::value_index(c, 4 * q)) >> 2;
+        ldsq_read128<0>(xq[q], lds_x + 16u * Q::swz(unit));
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int q = 0; q < 16; ++q) asm volatile("" : "+v"(xq[q]));
+#pragma unroll
+      for (int s = 0; s < Q::NSUM; ++s) sx[s] = 0.0f;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        f32x4 v = as_f32x4(xq[q]);
+        if (!valid) v = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        xr[4 * q + 0] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+        sx[Q::sum_index(4 * q)] += (v.x + v.y) + (v.z + v.w);
+      }
+    }
+    typename Q::Regs regs[U];
+    bool nxt_in_flight = true;
+    for (u32 it = 0; cur < batches; ++it) {
+      // batch `cur` has landed when at most the copies of the batch behind it are outstanding
+      if (nxt_in_flight) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const u32 slot = it & 1u;
+      const u32 base = lds_ring + slot * Slot::BYTES + shift_cur + sbc * Q::SB;
+#pragma unroll
+      for (int u = 0; u < U; ++u) Q::load_lds(regs[u], base + u * row_bytes, c);
+      // the batch after the next: handed out among the waves as they become free (the memory system does not serve
+      // them evenly); its copies go where the current batch was, which is in registers when the reads have returned
+      u32 nn;
+      asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nn) : "v"(lds_next), "v"(lane == 0 ? 1u : 0u) : "memory");
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int u = 0; u < U; ++u) Q::landed(regs[u]);
+      asm volatile("" : "+v"(nn));
+      nn = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(nn)));
+      const bool more = nn < batches;
+      u32 shift_nn = 0;
+      if (more) shift_nn = issue(nn, slot);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
+        if (lane == 0) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_part + 4u * (cur * U + u)), "v"(p) : "memory");
+      }
+      cur = nxt; shift_cur = shift_nxt;
+      nxt = nn; shift_nxt = shift_nn;
+      nxt_in_flight = more;
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // copies of batches that do not exist, partial sums
+  __syncthreads();
+  const float* part = reinterpret_cast<float*>(lds4 + units);
+  const float* group_ss = part + rows_per_block;
+  float scale = 1.0f;
+  if (norm) {
+    float total_ss = group_ss[0];
+    for (u32 g = 1; g < xgroups; ++g) total_ss += group_ss[g];
+    scale = 1.0f / sqrtf(total_ss / static_cast<float>(k_dim) + (e.eps != 0.0f ? e.eps : kChainNormEps));
+  }
+  for (u32 t = tid; t < rows_per_block; t += block_threads) {
+    const u32 row = row0 + t;
+    if (row < n_dim) {
+      float r = part[t] * scale;
+      if (e.residual) r = __fadd_rn(r, e.residual[row]);
+      e.y[row] = r;
+    }
+  }
+  return true;
+}
+
 // One entry on this workgroup's share of rows.  Returns false if the barrier wait gave up.
 //   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][k/256 group sums of squares]
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
@@ -123,6 +347,8 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
   // The engine is built for whole waves: a block that is not a positive multiple of 64 threads (the reference's own
   // geometry is 32) would divide by zero below and never leave the staging loop.  Uniform exit before any barrier.
   if (block_threads < 64u || (block_threads & 63u) != 0u) return true;
+  if constexpr (!COHERENT)      // (the resident executor keeps the register path: its launcher never sets the flag)
+    if ((e.flags & CHAIN_STREAM_LDS) && wait_counter == nullptr) return chain_step_stream<FMT, U>(e, lds4, block_id, num_blocks, block_threads);
   const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = block_threads >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;

@@ -161,9 +161,17 @@ __device__ __forceinline__ void convert_chunk(const f32x4& v0, const f32x4& v1, 
   // of a token, which write the same slot of different pages, do not all hit one bank (the reader applies the same)
   lds_write128x2(stage + q * 1024u + ((32u * g + 2u * token) ^ (2u * q)) * 16u, ph, pl);
   if constexpr (SUMS) {
-    float sj = ((xs[0] + xs[1]) + (xs[2] + xs[3])) + ((xs[4] + xs[5]) + (xs[6] + xs[7]));
-    sj += dpp_f32<0xB1>(sj);
-    sj += dpp_f32<0x4E>(sj);                // the four threads of a sub-block hold its sum
+    // The sub-block's sum is formed from the pieces, not from the f32 values: a piece has eleven significant bits, so
+    // thirty-two of them of similar size add up without rounding in f32, where the values themselves round at every
+    // step - and the sum is multiplied by C * s_j (the centring term of the Q4_K / Q5_K products), which is large.
+    const h16x2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+    float sh = __builtin_amdgcn_fdot2(as_h16x2(ph.x), ones, 0.0f, false), sl = __builtin_amdgcn_fdot2(as_h16x2(pl.x), ones, 0.0f, false);
+    sh = __builtin_amdgcn_fdot2(as_h16x2(ph.y), ones, sh, false); sl = __builtin_amdgcn_fdot2(as_h16x2(pl.y), ones, sl, false);
+    sh = __builtin_amdgcn_fdot2(as_h16x2(ph.z), ones, sh, false); sl = __builtin_amdgcn_fdot2(as_h16x2(pl.z), ones, sl, false);
+    sh = __builtin_amdgcn_fdot2(as_h16x2(ph.w), ones, sh, false); sl = __builtin_amdgcn_fdot2(as_h16x2(pl.w), ones, sl, false);
+    sh += dpp_f32<0xB1>(sh); sl += dpp_f32<0xB1>(sl);
+    sh += dpp_f32<0x4E>(sh); sl += dpp_f32<0x4E>(sl);      // the four threads of a sub-block hold its sums
+    const float sj = fmaf(sl, 0.00048828125f, sh);
     if ((c & 3u) == 0u) {
       _Float16 sh, sl;
       split_f16(sj * 0.03125f, sh, sl);
@@ -373,9 +381,13 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
                    : "=&v"(an[i][0]), "=&v"(an[i][1]) : "v"(src) : "memory");
     }
   };
-  auto convert = [&](u32 s) {          // the loads of A issued last have landed when DMA loads (of W) are left
+  // The loads of A issued last have landed when no more than the copies of W behind them are outstanding.  The last of
+  // those copies stands under `lane < 32`, which the compiler turns into a branch around it: on paper a wave can pass
+  // with DMA - 1 copies behind its loads of A, so that is the number waited for (it costs the first sixteenth of the
+  // weight tile having arrived as well).
+  auto convert = [&](u32 s) {
 #pragma unroll
-    for (int i = 0; i < NC; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA) : "memory");
+    for (int i = 0; i < NC; ++i) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(an[i][0]), "+v"(an[i][1]) : "n"(DMA - 1) : "memory");
     const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
     if (!converts) return;
 #pragma unroll
@@ -384,11 +396,14 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
                     ctoken[i], cpos[i], lds_xp + (s & 1u) * kStage + (i / CHUNKS) * kXpStageBytes);
   };
 
-  f32x16 tot[NT];
+  // Two running sums per result, for the even and the odd super-blocks of the run: each is half as long and half as
+  // large when it is rounded as one sum over all of them would be (the reference spreads a row over 32 lanes' sums,
+  // quantize.rs:1486, 1495-1508; here one register holds a whole row's).
+  f32x16 tot[NT], tot_odd[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) tot[t][v] = 0.0f;
+    for (int v = 0; v < 16; ++v) tot[t][v] = tot_odd[t][v] = 0.0f;
   u32 xq[16];                                    // where this lane finds its token operands of product q (stage 0)
 #pragma unroll
   for (u32 q = 0; q < 16; ++q) xq[q] = lds_xp + ((lane ^ (2u * q)) << 4);
@@ -430,10 +445,12 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
 #pragma unroll
     for (int t = 0; t < NT; ++t) asm volatile("" : "+v"(sx[t]), "+v"(f01[t]), "+v"(f23[t]), "+v"(f45[t]), "+v"(f67[t]));
     asm volatile("" : "+v"(qh));
-    if (s + 1u < ns) convert(s + 1u);        // into the stage that was read two super-blocks ago
-    if (s + 2u < ns) {          // the weight tile is in registers: its LDS space takes the tile after the next
-      load_a(s + 2u);
-      issue_w(s + 2u);
+    if (s + 1u < ns) {
+      convert(s + 1u);          // into the stage that was read two super-blocks ago
+      if (s + 2u < ns) {        // the weight tile is in registers: its LDS space takes the tile after the next
+        load_a(s + 2u);         // (inside the first condition: no path issues loads without having waited for the last ones)
+        issue_w(s + 2u);
+      }
     }
     const u32 dw[16] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w, d2.x, d2.y, d2.z, d2.w, d3.x, d3.y, d3.z, d3.w};
     const float d = half_bits_to_f32(hdr.x), dmin = half_bits_to_f32(hdr.x >> 16);
@@ -449,13 +466,25 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
       s4 = (f0 & 63u) | ((f1 & 63u) << 8) | ((f2 & 63u) << 16) | ((f3 & 63u) << 24);
       m4 = (f0 >> 6) | ((f1 >> 6) << 8) | ((f2 >> 6) << 16) | ((f3 >> 6) << 24);
     }
-    h16x2 sc[4];
+    // The quants enter centred: (q - C) * s_j with C = 8 (Q4_K) or 16 (Q5_K), and C * s_j * (sum of the sub-block's
+    // activations) is added by one small product at the end.  The running sums inside the matrix cores are then those of
+    // numbers spread around zero, about half as large as with q >= 0, and so are their rounding errors (measured:
+    // 1.2 times the error of an f32 evaluation in the reference's order uncentred; Q6_K, whose digits are centred by
+    // construction, 1.0).  (q - C) * s_j stays below 2048 in magnitude: exact in f16, as is the multiply-add that forms it.
+    constexpr float kCentre = FMT == FMT_Q4K ? 8.0f : 16.0f;
+    h16x2 sc[4], ad[4];
+    _Float16 sf[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const _Float16 sv = static_cast<_Float16>(static_cast<unsigned short>((s4 >> (8 * e)) & 0xFFu)) *
-                          static_cast<_Float16>((e & 1) ? 64.0f : 1024.0f);
+      sf[e] = static_cast<_Float16>(static_cast<unsigned short>((s4 >> (8 * e)) & 0xFFu));
+      const _Float16 sv = sf[e] * static_cast<_Float16>((e & 1) ? 64.0f : 1024.0f);
+      const _Float16 av = sf[e] * static_cast<_Float16>(-kCentre * 0.00006103515625f);      // -C * s_j * 2^-14
       sc[e] = h16x2{sv, sv};
+      ad[e] = h16x2{av, av};
     }
+    // C * s_j * 2^-9 against the sub-block sums (which carry 2^-5): C * s_j * 2^-14 * sum, the scale of the main products
+    const h16x4 cb = {sf[0] * static_cast<_Float16>(kCentre * 0.001953125f), sf[1] * static_cast<_Float16>(kCentre * 0.001953125f),
+                      sf[2] * static_cast<_Float16>(kCentre * 0.001953125f), sf[3] * static_cast<_Float16>(kCentre * 0.001953125f)};
     const h16x4 mb = {static_cast<_Float16>(static_cast<unsigned short>(m4 & 0xFFu)),
                       static_cast<_Float16>(static_cast<unsigned short>((m4 >> 8) & 0xFFu)),
                       static_cast<_Float16>(static_cast<unsigned short>((m4 >> 16) & 0xFFu)),
@@ -463,10 +492,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     f32x16 macc[NT], acc[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      macc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx[t]), mb, zero, 0, 0, 0);
-      acc[t] = zero;
-    }
+    for (int t = 0; t < NT; ++t) acc[t] = zero;
 #pragma unroll
     for (int uu = 0; uu < 8; uu += 2) {          // two dword pairs = four products per round of operand reads
       u32x4 ax[NT][4];
@@ -485,7 +511,7 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
       for (int i = 0; i < 2; ++i) {
         const int u = uu + i;
         const u32 t0 = dw[2 * u], t1 = dw[2 * u + 1], t0s = t0 >> 8, t1s = t1 >> 8;
-        const h16x2 sl2 = sc[(u >> 2) * 2], sh2 = sc[(u >> 2) * 2 + 1];
+        const h16x2 sl2 = sc[(u >> 2) * 2], sh2 = sc[(u >> 2) * 2 + 1], al2 = ad[(u >> 2) * 2], ah2 = ad[(u >> 2) * 2 + 1];
         // Q5_K: the fifth bits of the eight values of dword j (j = 2u, 2u+1) are nibble j%8 of qh word 2(j/8) (low
         // nibbles) and 2(j/8)+1 (high nibbles), bit i for byte i.  n * (2^4 + 2^18) puts bit 0 at bit 4 and bit 2 at
         // bit 20 - where the fifth bit of a low nibble's 16-bit lane belongs for bytes 0 and 2 -, n * (2^3 + 2^17) the
@@ -502,14 +528,14 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
             e[d][1] = __umul24(nh, 0x200080u) & 0x01000100u;     // high nibbles, bytes 1 and 3
           }
         }
-        bl[i][0] = __builtin_bit_cast(u32, pk_mul_h2((t0 & 0x000F000Fu) | f[0][0], sl2));
-        bl[i][1] = __builtin_bit_cast(u32, pk_mul_h2((t0s & 0x000F000Fu) | f[0][1], sl2));
-        bl[i][2] = __builtin_bit_cast(u32, pk_mul_h2((t1 & 0x000F000Fu) | f[1][0], sl2));
-        bl[i][3] = __builtin_bit_cast(u32, pk_mul_h2((t1s & 0x000F000Fu) | f[1][1], sl2));
-        bh[i][0] = __builtin_bit_cast(u32, pk_mul_h2((t0 & 0x00F000F0u) | e[0][0], sh2));
-        bh[i][1] = __builtin_bit_cast(u32, pk_mul_h2((t0s & 0x00F000F0u) | e[0][1], sh2));
-        bh[i][2] = __builtin_bit_cast(u32, pk_mul_h2((t1 & 0x00F000F0u) | e[1][0], sh2));
-        bh[i][3] = __builtin_bit_cast(u32, pk_mul_h2((t1s & 0x00F000F0u) | e[1][1], sh2));
+        bl[i][0] = __builtin_bit_cast(u32, pk_fma_h2((t0 & 0x000F000Fu) | f[0][0], sl2, al2));
+        bl[i][1] = __builtin_bit_cast(u32, pk_fma_h2((t0s & 0x000F000Fu) | f[0][1], sl2, al2));
+        bl[i][2] = __builtin_bit_cast(u32, pk_fma_h2((t1 & 0x000F000Fu) | f[1][0], sl2, al2));
+        bl[i][3] = __builtin_bit_cast(u32, pk_fma_h2((t1s & 0x000F000Fu) | f[1][1], sl2, al2));
+        bh[i][0] = __builtin_bit_cast(u32, pk_fma_h2((t0 & 0x00F000F0u) | e[0][0], sh2, ah2));
+        bh[i][1] = __builtin_bit_cast(u32, pk_fma_h2((t0s & 0x00F000F0u) | e[0][1], sh2, ah2));
+        bh[i][2] = __builtin_bit_cast(u32, pk_fma_h2((t1 & 0x00F000F0u) | e[1][0], sh2, ah2));
+        bh[i][3] = __builtin_bit_cast(u32, pk_fma_h2((t1s & 0x00F000F0u) | e[1][1], sh2, ah2));
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) lds_wait4(ax[t][0], ax[t][1], ax[t][2], ax[t][3]);
@@ -524,19 +550,34 @@ __device__ __forceinline__ void kq_body(const float* __restrict__ a, const uint8
           acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, ax[t][2 * i + 1]), __builtin_bit_cast(h16x8, bhv), acc[t], 0, 0, 0);
       }
     }
+    // what the centring took out, added to the main products in one step; then the min term's product (last: its
+    // sixteen results per tile are not alive while the main products run)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx[t]), cb, acc[t], 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) macc[t] = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(h16x4, sx[t]), mb, zero, 0, 0, 0);
     const float nm = dmin * -0.001953125f;       // -dmin * 2^-9: the sums carry 2^-5, the products 2^-14
+    // the super-block's own term is formed first (it is small), then added: one rounding at the size of the running sum
+    // and the two running sums change places, so that each takes every other super-block
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const float fac[8] = {__uint_as_float(f01[t].x), __uint_as_float(f01[t].y), __uint_as_float(f23[t].x), __uint_as_float(f23[t].y),
                             __uint_as_float(f45[t].x), __uint_as_float(f45[t].y), __uint_as_float(f67[t].x), __uint_as_float(f67[t].y)};
+      const f32x16 other = tot[t];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float fd = fac[e] * d, fm = fac[e] * nm;
-        tot[t][2 * e] = fmaf(fm, macc[t][2 * e], fmaf(fd, acc[t][2 * e], tot[t][2 * e]));
-        tot[t][2 * e + 1] = fmaf(fm, macc[t][2 * e + 1], fmaf(fd, acc[t][2 * e + 1], tot[t][2 * e + 1]));
+        tot[t][2 * e] = tot_odd[t][2 * e] + fmaf(fm, macc[t][2 * e], fd * acc[t][2 * e]);
+        tot[t][2 * e + 1] = tot_odd[t][2 * e + 1] + fmaf(fm, macc[t][2 * e + 1], fd * acc[t][2 * e + 1]);
       }
+      tot_odd[t] = other;
     }
   }
+  // nothing is outstanding here (the last round waited for everything); said once more for the code that follows, which
+  // takes over the registers of the loads written in asm
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int t = 0; t < NT; ++t) tot[t] += tot_odd[t];
 
   finish_tiles<NT>(tot, c, ws, m, n, kparts, groups, tiles, tgroups, waves, group, part, tg, strip, col, g, lane, lds_flag);
 }
@@ -643,9 +684,12 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
       convert_chunk<false>(live[i] ? an[i][0] : zero4, live[i] ? an[i][1] : zero4, ctoken[i], cpos[i], lds_xp + (s & 1u) * kXpStageBytes);
   };
 
-  f32x16 tot;
+  // running sums over the even and the odd super-blocks (as in kq_body) where the registers allow it: the kernel of 4
+  // strips converts twice the tokens per thread and is at the limit of two waves per SIMD with one sum
+  constexpr bool kTwoSums = CHUNKS == 1;
+  f32x16 tot, tot_odd;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) tot[v] = 0.0f;
+  for (int v = 0; v < 16; ++v) tot[v] = tot_odd[v] = 0.0f;
   u32 xq[16];                                    // where this lane finds its token operands of page Q (stage 0)
 #pragma unroll
   for (u32 q = 0; q < 16; ++q) xq[q] = lds_xp + ((lane ^ (2u * q)) << 4);
@@ -744,15 +788,17 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
     if constexpr (NEXT2) load_w(s + 2u);
     const float fac[8] = {__uint_as_float(f01.x), __uint_as_float(f01.y), __uint_as_float(f23.x), __uint_as_float(f23.y),
                           __uint_as_float(f45.x), __uint_as_float(f45.y), __uint_as_float(f67.x), __uint_as_float(f67.y)};
+    const f32x16 other = tot;                    // the two running sums change places: each takes every other super-block
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const float fd = fac[t] * d;
 #pragma unroll
       for (int pc = 0; pc < 2; ++pc) {
         const int v = 2 * t + pc;
-        tot[v] = fmaf(fd, fmaf(8.0f, acc_q[v], acc_n[v]), tot[v]);
+        tot[v] = fmaf(fd, fmaf(8.0f, acc_q[v], acc_n[v]), kTwoSums ? tot_odd[v] : tot[v]);
       }
     }
+    if constexpr (kTwoSums) tot_odd = other;
   };
   using std::true_type;
   using std::false_type;
@@ -771,7 +817,7 @@ __device__ __forceinline__ void q6k_body(const float* __restrict__ a, const uint
     step(s, true_type{}, false_type{});
     step(s + 1u, false_type{}, false_type{});
   }
-  const f32x16 tots[1] = {tot};
+  const f32x16 tots[1] = {tot + tot_odd};
   finish_tiles<1>(tots, c, ws, m, n, kparts, groups, tiles, tiles, waves, group, part, tile, strip, col, g, lane, lds_flag);
 }
 

@@ -16,6 +16,22 @@
 
 template <int FMT> struct Quarter;
 
+// LDS reads written in asm: a row batch streamed into LDS by DMA is still arriving while the previous one is read, and
+// for LDS accesses the compiler can see it waits until every such copy has landed.  The caller waits (lgkmcnt) and then
+// passes the registers through landed().
+template <int OFF> __device__ __forceinline__ void ldsq_read128(u32x4& v, u32 addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF> __device__ __forceinline__ void ldsq_read64(u32x2& v, u32 addr) {
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF> __device__ __forceinline__ void ldsq_read32(u32& v, u32 addr) {
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF> __device__ __forceinline__ void ldsq_read16(u32& v, u32 addr) {
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=&v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+
 // ------------------------------------------------------------------------------------------
 // Q4_K: quarter c holds qs[32c .. 32c+31]; low nibbles are values 64c+0..31 (sub-block 2c),
 // high nibbles are values 64c+32..63 (sub-block 2c+1).
@@ -34,6 +50,14 @@ template <> struct Quarter<FMT_Q4K> {
     r.q0 = load128(sbp + 16 + 32 * c);
     r.q1 = load128(sbp + 32 + 32 * c);
   }
+
+  // the same three pieces from a copy of the block in LDS (at byte address `blk`)
+  static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {
+    ldsq_read128<0>(r.hdr, blk);
+    ldsq_read128<16>(r.q0, blk + 32u * c);
+    ldsq_read128<32>(r.q1, blk + 32u * c);
+  }
+  static __device__ __forceinline__ void landed(Regs& r) { asm volatile("" : "+v"(r.hdr), "+v"(r.q0), "+v"(r.q1)); }
 
   // (d*s, dmin*m) for sub-blocks 2c and 2c+1; get_scale_min_k4 packing (quantize.rs:1306-1385).
   static __device__ __forceinline__ void scales(const Regs& r, u32 c, float& ds0, float& ds1, float& dm0, float& dm1) {
@@ -61,24 +85,29 @@ template <> struct Quarter<FMT_Q4K> {
   static __device__ __forceinline__ float dot(const Regs& r, u32 c, const float (&xr)[64], const float (&sx)[NSUM]) {
     float ds0, ds1, dm0, dm1;
     scales(r, c, ds0, ds1, dm0, dm1);
-    float lo = 0.0f, hi = 0.0f;  // lo accumulates 2^-24 * q x, hi 2^-20 * q x
+    // Each sub-block's 32 products go into four chains of eight, joined pairwise: no chain is longer than the
+    // reference's (eight FMAs per lane and super-block, quantize.rs:1412, 1482), so no partial sum grows larger
+    // before it is rounded.  lo accumulates 2^-24 * q x, hi 2^-20 * q x.
+    float lo[4] = {0.0f, 0.0f, 0.0f, 0.0f}, hi[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const u32 v = t < 4 ? r.q0[t] : r.q1[t - 4];
       const u32 w = v >> 8;
       const h16x2 l02 = as_h16x2(v & 0x000F000Fu), h02 = as_h16x2(v & 0x00F000F0u);   // bytes 0 and 2
       const h16x2 l13 = as_h16x2(w & 0x000F000Fu), h13 = as_h16x2(w & 0x00F000F0u);   // bytes 1 and 3
-      lo = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], lo);
-      lo = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], lo);
-      lo = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], lo);
-      lo = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], lo);
-      hi = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], hi);
-      hi = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], hi);
-      hi = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], hi);
-      hi = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], hi);
+      float& l = lo[t & 3];
+      float& h = hi[t & 3];
+      l = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], l);
+      l = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], l);
+      l = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], l);
+      l = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], l);
+      h = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], h);
+      h = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], h);
+      h = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], h);
+      h = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], h);
     }
-    float acc = (ds0 * 16777216.0f) * lo;
-    acc = fmaf(ds1 * 1048576.0f, hi, acc);
+    float acc = (ds0 * 16777216.0f) * ((lo[0] + lo[1]) + (lo[2] + lo[3]));
+    acc = fmaf(ds1 * 1048576.0f, (hi[0] + hi[1]) + (hi[2] + hi[3]), acc);
     acc = fmaf(-dm0, sx[0], acc);
     acc = fmaf(-dm1, sx[1], acc);
     return acc;
@@ -122,6 +151,15 @@ template <> struct Quarter<FMT_Q5K> {
     r.qh = load64(sbp + 144 + 8 * c);
   }
 
+  static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {
+    ldsq_read32<0>(r.dd, blk);
+    ldsq_read32<4>(r.f24, blk + 3u * c);         // at any byte alignment, like the load from memory
+    ldsq_read128<16>(r.q0, blk + 32u * c);
+    ldsq_read128<32>(r.q1, blk + 32u * c);
+    ldsq_read64<144>(r.qh, blk + 8u * c);
+  }
+  static __device__ __forceinline__ void landed(Regs& r) { asm volatile("" : "+v"(r.dd), "+v"(r.f24), "+v"(r.q0), "+v"(r.q1), "+v"(r.qh)); }
+
   static __device__ __forceinline__ void scales(const Regs& r, float& ds0, float& ds1, float& dm0, float& dm1) {
     const float d = half_bits_to_f32(r.dd);
     const float dmin = half_bits_to_f32(r.dd >> 16);
@@ -143,7 +181,7 @@ template <> struct Quarter<FMT_Q5K> {
   static __device__ __forceinline__ float dot(const Regs& r, u32 c, const float (&xr)[64], const float (&sx)[NSUM]) {
     float ds0, ds1, dm0, dm1;
     scales(r, ds0, ds1, dm0, dm1);
-    float lo = 0.0f, hi = 0.0f;
+    float lo[4] = {0.0f, 0.0f, 0.0f, 0.0f}, hi[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // four chains of eight per sub-block, as for Q4_K
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const u32 v = t < 4 ? r.q0[t] : r.q1[t - 4];
@@ -153,17 +191,19 @@ template <> struct Quarter<FMT_Q5K> {
       const u32 h = opaque(join5((v >> 4) & 0x0F0F0F0Fu, bh));
       const h16x2 l02 = as_h16x2(l & 0x001F001Fu), l13 = as_h16x2((l >> 8) & 0x001F001Fu);   // bytes 0,2 and 1,3
       const h16x2 h02 = as_h16x2(h & 0x001F001Fu), h13 = as_h16x2((h >> 8) & 0x001F001Fu);
-      lo = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], lo);
-      lo = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], lo);
-      lo = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], lo);
-      lo = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], lo);
-      hi = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], hi);
-      hi = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], hi);
-      hi = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], hi);
-      hi = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], hi);
+      float& lc = lo[t & 3];
+      float& hc = hi[t & 3];
+      lc = fmaf(static_cast<float>(l02.x), xr[4 * t + 0], lc);
+      lc = fmaf(static_cast<float>(l13.x), xr[4 * t + 1], lc);
+      lc = fmaf(static_cast<float>(l02.y), xr[4 * t + 2], lc);
+      lc = fmaf(static_cast<float>(l13.y), xr[4 * t + 3], lc);
+      hc = fmaf(static_cast<float>(h02.x), xr[32 + 4 * t + 0], hc);
+      hc = fmaf(static_cast<float>(h13.x), xr[32 + 4 * t + 1], hc);
+      hc = fmaf(static_cast<float>(h02.y), xr[32 + 4 * t + 2], hc);
+      hc = fmaf(static_cast<float>(h13.y), xr[32 + 4 * t + 3], hc);
     }
-    float acc = (ds0 * 16777216.0f) * lo;
-    acc = fmaf(ds1 * 16777216.0f, hi, acc);
+    float acc = (ds0 * 16777216.0f) * ((lo[0] + lo[1]) + (lo[2] + lo[3]));
+    acc = fmaf(ds1 * 16777216.0f, (hi[0] + hi[1]) + (hi[2] + hi[3]), acc);
     acc = fmaf(-dm0, sx[0], acc);
     acc = fmaf(-dm1, sx[1], acc);
     return acc;
@@ -216,6 +256,16 @@ template <> struct Quarter<FMT_Q6K> {
     r.sc = load64_a2(sbp + 192 + 8 * h);
     r.d = load16_a2(sbp + 208);
   }
+
+  static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {       // blocks lie at 2-byte alignment in LDS too
+    const u32 h = c >> 1, is = c & 1u;
+    ldsq_read128<0>(r.a, blk + 64u * h + 16u * is);
+    ldsq_read128<32>(r.b, blk + 64u * h + 16u * is);
+    ldsq_read128<128>(r.c, blk + 32u * h + 16u * is);
+    ldsq_read64<192>(r.sc, blk + 8u * h);
+    ldsq_read16<208>(r.d, blk);
+  }
+  static __device__ __forceinline__ void landed(Regs& r) { asm volatile("" : "+v"(r.a), "+v"(r.b), "+v"(r.c), "+v"(r.sc), "+v"(r.d)); }
 
   static __device__ __forceinline__ void scales(const Regs& r, u32 c, float (&dsc)[4]) {
     const float d = half_bits_to_f32(r.d);

@@ -62,6 +62,12 @@ constexpr uint32_t kGemvRowsPerBatch = KQ_U;  // U of the fast GEMV kernel (the 
 constexpr uint32_t kGemvMaxWaves = 12;        // __launch_bounds__(768) of the fast GEMV kernels
 constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels may ask for
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
+// The engine for matrices of one slab (k <= 4096) streams the rows through LDS (chain_step_stream of kquant_chain.hip.h):
+// behind the vector, the partial sums and the scratch every wave owns a ring of two slots of this many bytes (a batch of
+// KQ_U rows of 16 blocks, from the 16-byte boundary below its first byte, in whole KB: StreamSlot of the kernels).
+constexpr uint32_t kChainStreamFlag = 16u;     // CHAIN_STREAM_LDS
+constexpr uint32_t kStreamLdsLimit = 160 * 1024 - 1024;   // dynamic LDS such a launch may ask for (the CU has 160 KB; static LDS is a few words)
+constexpr uint32_t stream_slot_bytes(uint32_t sb_bytes) { return (kGemvRowsPerBatch * 16u * sb_bytes + 15u + 1023u) / 1024u * 1024u; }
 
 struct DeviceKernels {
   bool loaded = false;
@@ -103,6 +109,8 @@ std::atomic<int> g_tune_group_max{0};          // most entries in one grouped la
 std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
 std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4, 8 or (Q4_K) 12 (0: default)
+std::atomic<int> g_tune_stream_off{0};      // 1: one-slab GEMVs load their rows into registers straight from memory (no LDS ring)
+std::atomic<int> g_tune_stream_waves{0};    // waves per workgroup of a single streamed GEMV (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -198,6 +206,31 @@ struct GemvGeometry {
   uint32_t grid = 0, block = 0, lds = 0;
   bool fits = false;
 };
+
+// Can an n x k matrix of this format go through the streamed engine?  (one slab; any alignment the fast kernels take)
+bool stream_ok(uint32_t k) { return !g_tune_stream_off && k != 0 && k <= 4096u; }
+
+// Geometry of a single streamed GEMV: workgroups of `waves` waves, as many per CU as their LDS allows (two by default).
+GemvGeometry stream_geometry(const DeviceKernels& d, Fmt f, uint32_t k, uint32_t n) {
+  GemvGeometry g;
+  const uint32_t waves = g_tune_stream_waves > 0 ? std::min<uint32_t>(uint32_t(g_tune_stream_waves), kGemvMaxWaves) : 4u;
+  const uint32_t ring = waves * 2u * stream_slot_bytes(kSbBytes[f]);
+  const uint64_t fixed = uint64_t(k) * 4u + kLdsScratch + ring;
+  if (fixed + kGemvRowsPerBatch * 4u > kStreamLdsLimit) return g;
+  const uint32_t fit = uint32_t(std::max<uint64_t>(1, (160u * 1024u) / (fixed + 1024u)));
+  const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::min(fit, std::max(1u, 8u / waves));
+  const uint64_t target_blocks = uint64_t(d.cu_count) * per_cu;
+  const uint32_t ug = kGemvRowsPerBatch;
+  uint64_t rows = (uint64_t(n) + target_blocks - 1) / target_blocks;
+  rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
+  const uint64_t max_rows = (kStreamLdsLimit - fixed) / 4u / ug * ug;
+  rows = std::min<uint64_t>(rows, max_rows);
+  g.grid = uint32_t((uint64_t(n) + rows - 1) / rows);
+  g.block = 64u * waves;
+  g.lds = uint32_t(fixed + rows * 4u);
+  g.fits = true;
+  return g;
+}
 
 GemvGeometry gemv_geometry(const DeviceKernels& d, uint32_t k, uint32_t n, uint32_t max_waves = kGemvMaxWaves) {
   GemvGeometry g;
@@ -524,6 +557,13 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void* gemm_args[] = {&a, &w, &c, &m, &n, &k};
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
+  if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(k)) {
+    g = stream_geometry(*d, f, k, n);
+    if (g.fits) {
+      flags |= kChainStreamFlag;
+      return hipModuleLaunchKernel(d->gemv_flags[f], g.grid, 1u, 1, g.block, 1, 1, g.lds, stream, args, nullptr);
+    }
+  }
   if (k != 0 && gemv_fast_ok(f, c, w, a) && (is_gemv || (aligned(uint64_t(k) * 4u, 16) && aligned(uint64_t(n) * 4u, 4))))
     g = gemv_geometry(*d, k, n, is_gemv ? kGemvMaxWaves : 8u);   // the GEMM kernels are built for 8 waves
   if (g.fits) {
@@ -1325,18 +1365,27 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   uint32_t first[kGroupMax + 1] = {};
   uint32_t lds = 0;
   // rows per workgroup and workgroups of entry i when it is given `share` workgroups (0 rows: it does not fit the engine)
+  // an entry of one slab streams its rows through LDS when the rings of all waves fit beside its vector
+  auto ring_of = [&](uint32_t i) -> uint32_t {
+    const trn_gemv_desc& e = descs[i];
+    if (!stream_ok(e.k)) return 0u;
+    const uint32_t ring = waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]);
+    return uint64_t(e.k) * 4u + kLdsScratch + ring + kGemvRowsPerBatch * 4u <= kStreamLdsLimit ? ring : 0u;
+  };
   struct Cut { uint64_t rows; uint32_t grid; };
   auto cut_of = [&](uint32_t i, uint64_t share) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves), groups = waves / sw;
     const uint64_t x_bytes = uint64_t(e.k) * 4u;
-    // workgroups of 8 waves or more hand their row batches out among the waves: a share need not be a whole
-    // number of rounds of all waves
-    const uint32_t ug = waves >= 8u ? kGemvRowsPerBatch : kGemvRowsPerBatch * groups;
+    const uint32_t ring = ring_of(i);
+    const uint64_t limit = ring ? kStreamLdsLimit - ring : kFastLdsLimit;
+    // workgroups of 8 waves or more (and every streamed entry) hand their row batches out among the waves: a share
+    // need not be a whole number of rounds of all waves
+    const uint32_t ug = (waves >= 8u || ring) ? kGemvRowsPerBatch : kGemvRowsPerBatch * groups;
     uint64_t rows = (uint64_t(e.n) + share - 1) / share;
     rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
-    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > kFastLdsLimit) return Cut{0u, 0u};
-    const uint64_t max_rows = (kFastLdsLimit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
+    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > limit) return Cut{0u, 0u};
+    const uint64_t max_rows = (limit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug;
     rows = std::min<uint64_t>(rows, max_rows);
     return Cut{rows, uint32_t((uint64_t(e.n) + rows - 1) / rows)};
   };
@@ -1386,9 +1435,10 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   for (uint32_t i = 0; i < len; ++i) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t nsb = e.k / 256u, slabs = (nsb + 15u) / 16u, sw = std::min(slabs, waves);
-    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags, 0u, 0u};
+    const uint32_t ring = ring_of(i);
+    g.hot[i] = {e.w, e.x, e.k, e.n, e.fmt, e.flags | (ring ? kChainStreamFlag : 0u), 0u, 0u};
     g.cold[i] = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
-    lds = std::max<uint32_t>(lds, uint32_t(uint64_t(e.k) * 4u + uint64_t(sw) * cut[i].rows * 4u + kLdsScratch));
+    lds = std::max<uint32_t>(lds, uint32_t(uint64_t(e.k) * 4u + uint64_t(sw) * cut[i].rows * 4u + kLdsScratch + ring));
     first[i + 1] = first[i] + cut[i].grid;
     g.hot[i].first_block = first[i];
     g.hot[i].num_blocks = cut[i].grid;
@@ -1639,6 +1689,8 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "group_slab_weight")) { g_tune_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_per_cu")) { g_tune_attention_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "attention_min_steps")) { g_tune_attention_min_steps = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemv_stream_off")) { g_tune_stream_off = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemv_stream_waves")) { g_tune_stream_waves = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
