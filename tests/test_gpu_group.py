@@ -113,10 +113,11 @@ def test_grouped_equals_separate(gpu, case):
         assert kq.rel_l2(got[dst], ref) <= TOL, (case, dst)
 
 
-@pytest.mark.parametrize("group_max", (0, 11, 8))
-def test_up_to_sixteen_entries_in_one_launch(gpu, group_max):
-    """Nineteen independent entries of mixed formats and shapes: by default sixteen to a launch (every position of the
-    kernel's table of first workgroups is used), fewer with "group_max".  Same bits as one launch per entry."""
+@pytest.mark.parametrize("group_max", (0, 16, 11, 8))
+def test_nineteen_independent_entries(gpu, group_max):
+    """Nineteen independent entries of mixed formats and shapes: by default all in one launch (more than sixteen: the
+    launch that takes its entries from tables in device memory), with "group_max" sixteen to a launch (every position of
+    the kernel-argument table of first workgroups is used) or fewer.  Same bits as one launch per entry."""
     fmts = ("q4k", "q5k", "q6k")
     specs = [(fmts[i % 3], 33 + 41 * i, 256 * (1 + (i * 5) % 7), "x", f"y{i}", i % 2) for i in range(19)]
     sep, _ = _run(gpu, specs, 256 * 7, 1)
@@ -128,7 +129,7 @@ def test_up_to_sixteen_entries_in_one_launch(gpu, group_max):
     finally:
         _tune("group_max", 0)
         _tune("group_window", 0)
-    most = {0: 16, 11: 11, 8: 8}[group_max]
+    most = {0: 19, 16: 16, 11: 11, 8: 8}[group_max]
     assert len(plan) == 19 and max(np.bincount(plan)) == most and max(plan) + 1 == -(-19 // most), plan
     for name in sep:
         assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), (group_max, name)
@@ -138,6 +139,66 @@ def test_up_to_sixteen_entries_in_one_launch(gpu, group_max):
         if flags:
             ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
         assert kq.rel_l2(got[dst], ref) <= TOL, (group_max, dst)
+
+
+@pytest.mark.parametrize("seed", (0, 1))
+def test_many_entries_in_one_launch(gpu, seed):
+    """Seventy independent entries - three formats, one to four slabs of columns, ragged and large row counts, with and
+    without the normalised input - go into ONE launch whose workgroups each take pieces of several entries (or a slice
+    of a large one).  Same bits as one launch per entry; every entry against fp64; a second call (the cached plan) and
+    a call after the list has changed give the same again."""
+    rng = np.random.default_rng(seed)
+    ks = (256, 1024, 4096, 4352, 8192, 11008, 14336)
+    ns = (1, 37, 300, 1024, 2817, 4096, 9000)
+    specs = [(("q4k", "q5k", "q6k")[int(rng.integers(3))], int(rng.choice(ns)), int(rng.choice(ks)), "x", f"y{i}", int(rng.integers(2)))
+             for i in range(70)]
+    sep, _ = _run(gpu, specs, 14336, 1)
+    plan = []
+    got, mats = _run(gpu, specs, 14336, 0, plan)
+    assert max(plan) == 0, plan                     # one launch
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), (seed, name)
+    for (fmt, n, k, src, dst, flags), m in zip(specs, mats):
+        x = got[src][:k].astype(np.float64)
+        ref = kq.dequant_matrix(fmt, m, n, k).astype(np.float64) @ x
+        if flags:
+            ref = ref / np.sqrt(np.mean(x * x) + 1e-6)
+        assert kq.rel_l2(got[dst], ref) <= TOL, (seed, dst, fmt, n, k)
+
+
+def test_many_entries_plan_is_reused_and_replaced(gpu):
+    """The cut of a list and its device tables are kept per stream for as long as the same list comes again; another list
+    replaces them.  Two lists issued alternately on one stream, each twice in a row: always the bits of one launch per entry."""
+    ctx, stream = gpu
+    lists = []
+    for li in range(2):
+        specs = [(("q4k", "q6k", "q5k")[(i + li) % 3], 200 + 37 * i, 256 * (1 + (i + li) % 5), "x", f"y{i}", i % 2) for i in range(24 + 6 * li)]
+        x = t.GpuBuffer.from_host(ctx, kq.gen_x(3 + li, 256 * 5))
+        outs, keep, batch = [], [], t.GemvBatch()
+        for i, (fmt, n, k, _, _, flags) in enumerate(specs):
+            w = t.GpuBuffer.from_host(ctx, kq.gen_matrix(fmt, 3000 + 100 * li + i, n, k))
+            y = t.GpuBuffer.from_host(ctx, np.full(n, np.nan, np.float32))
+            keep.append(w)
+            outs.append(y)
+            batch.add(fmt, k, n, y, w, x, flags)
+        _tune("group_off", 1)
+        try:
+            batch.launch(stream)
+            stream.synchronize()
+        finally:
+            _tune("group_off", 0)
+        want = [y.copy_to_host() for y in outs]
+        assert max(batch.plan()) == 0
+        lists.append((batch, outs, want, keep, x))
+    for rep in range(3):
+        for batch, outs, want, _, _ in lists:
+            for again in range(2):
+                for y, w0 in zip(outs, want):
+                    y.copy_from_host(np.full(len(w0), np.nan, np.float32))
+                batch.launch(stream)
+                stream.synchronize()
+                for i, (y, w0) in enumerate(zip(outs, want)):
+                    assert np.array_equal(y.copy_to_host().view(np.uint32), w0.view(np.uint32)), (rep, again, i)
 
 
 @pytest.mark.parametrize("seed", (0, 1, 2, 3))

@@ -130,8 +130,8 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
 //
 // A batch may start at any even address (Q6_K rows of 210-byte blocks): the copy starts at the 16-byte boundary below it
 // and the reads are shifted by the difference.  Pieces beyond the end of the batch (or of the matrix) repeat its last
-// piece: every wave instruction is issued unconditionally, so the number of copies outstanding is known where the waits
-// are written (vmcnt counted by hand; all LDS traffic in asm, see kquant_quarter.hip.h).
+// piece: a batch is always the same number of wave instructions, so the number of copies outstanding is known where
+// the waits are written (vmcnt counted by hand; all LDS traffic in asm, see kquant_quarter.hip.h).
 //   LDS: [k floats of x, swizzled][rows_per_block partial sums][64 group sums of squares][ring: waves * 2 * slot bytes]
 // ------------------------------------------------------------------------------------------------------------
 template <int FMT, int U> struct StreamSlot {
@@ -148,16 +148,13 @@ __device__ __forceinline__ void dma16_nt(const uint8_t* src, u32 lds_addr) {
 }
 
 template <int FMT, int U>
-__device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* lds4, u32 block_id, u32 num_blocks, u32 block_threads) {
+__device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* lds4, u32 row0, u32 rows_per_block, u32 block_threads) {
   using Q = Quarter<FMT>;
   using Slot = StreamSlot<FMT, U>;
   constexpr u32 NL = Slot::PIECES;
   const u32 tid = threadIdx.x, lane = tid & 63u, waves = block_threads >> 6;
   const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(tid >> 6)));
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;            // 1 <= nsb <= 16
-  u32 rows_per_block = (n_dim + num_blocks - 1) / num_blocks;
-  rows_per_block = ((rows_per_block + U - 1) / U) * U;
-  const u32 row0 = block_id * rows_per_block;
   if (row0 >= n_dim) return true;                                  // the whole workgroup: nothing was touched yet
   const u32 batches = rows_per_block / U;
   const u32 sbl = lane >> 2, c = lane & 3u;
@@ -173,15 +170,21 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
   __shared__ u32 s_next_stream;
   const u32 lds_next = lds_addr_of(&s_next_stream);
 
-  // batch b of this workgroup into ring slot `slot`; returns the byte shift of the batch inside the slot
+  // Batch b of this workgroup into ring slot `slot`; returns the byte shift of the batch inside the slot.
+  // Wave instruction j copies the 64 pieces 64 j .. 64 j + 63 of the batch; pieces behind the last byte of the batch
+  // repeat its last piece (the bytes behind a matrix need not exist), and a batch that does not exist is NL times the
+  // first piece of the matrix (one line, from the cache).  One form for every case, so that a batch is the same
+  // number of copies on every path: a branch between forms is two branches in the assembly, with a path that takes
+  // neither as far as a reader of the assembly can tell.
   auto issue = [&](u32 b, u32 slot) -> u32 {
     size_t off = static_cast<size_t>(row0 + b * U) * row_bytes;
-    if (off >= total) off = 0;                                       // a batch that does not exist: any valid bytes
+    const bool exists = b < batches && off < total;
+    if (!exists) off = 0;
     const u32 avail = static_cast<u32>(total - off < batch_bytes ? total - off : batch_bytes);
     const uint8_t* src = e.w + off;
     const u32 shift = static_cast<u32>(reinterpret_cast<size_t>(src)) & 15u;
     src -= shift;
-    const u32 last = (shift + avail - 1u) >> 4;                      // the last 16-byte piece that holds bytes of the batch
+    const u32 last = exists ? (shift + avail - 1u) >> 4 : 0u;       // the last 16-byte piece that holds bytes of the batch
     const u32 dst = lds_ring + slot * Slot::BYTES;
 #pragma unroll
     for (u32 j = 0; j < NL; ++j) {
@@ -191,8 +194,8 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
     return shift;
   };
 
-  // Activations first (loads return in order, and the vector is an L2 hit), then the first two batches of this wave,
-  // all unconditionally.  The loads of the vector are written in asm like the copies' waits: the compiler, which knows
+  // Activations first (loads return in order, and the vector is an L2 hit), then the first two batches of this wave.
+  // The loads of the vector are written in asm like the copies' waits: the compiler, which knows
   // the copies only as memory operations that write LDS, would wait for all of them before it touches LDS at all.
   constexpr u32 kXPre = 4;
   const bool swiglu = (e.flags & CHAIN_SWIGLU_INPUT) != 0u;
@@ -212,11 +215,13 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
     }
   }
   u32 cur = wave, nxt = wave + waves;
-  u32 shift_cur = issue(cur, 0u);
-  u32 shift_nxt = issue(nxt, 1u);
+  bool nxt_in_flight = true;
+  const u32 shift_cur0 = issue(cur, 0u), shift_nxt0 = issue(nxt, 1u);      // unconditionally: see issue
+  u32 shift_cur = shift_cur0, shift_nxt = shift_nxt0;
   // the vector has landed when only the copies issued behind it are outstanding
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
 #pragma unroll
-  for (u32 i = 0; i < kXPre; ++i) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xv[i]) : "n"(2 * NL) : "memory");
+  for (u32 i = 0; i < kXPre; ++i) asm volatile("" : "+v"(xv[i])::"memory");
   if (swiglu) {
 #pragma unroll
     for (u32 i = 0; i < kXPre; ++i) asm volatile("" : "+v"(x2v[i]));
@@ -284,7 +289,6 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       }
     }
     typename Q::Regs regs[U];
-    bool nxt_in_flight = true;
     for (u32 it = 0; cur < batches; ++it) {
       // batch `cur` has landed when at most the copies of the batch behind it are outstanding
       if (nxt_in_flight) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
@@ -315,7 +319,7 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       nxt_in_flight = more;
     }
   }
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // copies of batches that do not exist, partial sums
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // the copies of batches that do not exist; the partial sums
   __syncthreads();
   const float* part = reinterpret_cast<float*>(lds4 + units);
   const float* group_ss = part + rows_per_block;
@@ -340,23 +344,22 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
 //   LDS: [k floats of x, swizzled][sw_count * rows_per_block partial sums][k/256 group sums of squares]
 // COHERENT: x may have been written, and y may be read, by other workgroups of this same launch.
 // block_threads: blockDim.x, handed in by the kernel (an implicit kernel argument, i.e. a load: the kernel decides when).
+// chain_step_rows: the workgroup's rows are row0 .. row0 + rows_per_block - 1 (rows_per_block a multiple of U; rows
+// beyond the matrix are skipped).  chain_step: block block_id of num_blocks equal blocks of rows.
 template <int FMT, int U, bool COHERENT = false>
-__device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
-                                           f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks, u32 block_threads) {
+__device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
+                                                f32x4* lds4, u32* s_flag, u32 row0, u32 rows_per_block, u32 block_threads) {
   using Q = Quarter<FMT>;
   // The engine is built for whole waves: a block that is not a positive multiple of 64 threads (the reference's own
   // geometry is 32) would divide by zero below and never leave the staging loop.  Uniform exit before any barrier.
   if (block_threads < 64u || (block_threads & 63u) != 0u) return true;
   if constexpr (!COHERENT)      // (the resident executor keeps the register path: its launcher never sets the flag)
-    if ((e.flags & CHAIN_STREAM_LDS) && wait_counter == nullptr) return chain_step_stream<FMT, U>(e, lds4, block_id, num_blocks, block_threads);
+    if ((e.flags & CHAIN_STREAM_LDS) && wait_counter == nullptr) return chain_step_stream<FMT, U>(e, lds4, row0, rows_per_block, block_threads);
   const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = block_threads >> 6;
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;
   const u32 sw_count = slabs < waves ? slabs : waves;
   const u32 groups = waves / sw_count;
-  u32 rows_per_block = (n_dim + num_blocks - 1) / num_blocks;
-  rows_per_block = ((rows_per_block + U - 1) / U) * U;
-  const u32 row0 = block_id * rows_per_block;
   const bool has_rows = row0 < n_dim && nsb != 0;
   const u32 batches = has_rows ? rows_per_block / U : 0u;
   const u32 sw = wave % sw_count, grp = wave / sw_count;
@@ -521,6 +524,15 @@ __device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counte
     }
   }
   return true;
+}
+
+template <int FMT, int U, bool COHERENT = false>
+__device__ __forceinline__ bool chain_step(const ChainEntry& e, u32* wait_counter, u32 spin_limit, u32* status,
+                                           f32x4* lds4, u32* s_flag, u32 block_id, u32 num_blocks, u32 block_threads) {
+  u32 rows_per_block = (e.n + num_blocks - 1) / num_blocks;
+  rows_per_block = ((rows_per_block + U - 1) / U) * U;
+  return chain_step_rows<FMT, U, COHERENT>(e, wait_counter, spin_limit, status, lds4, s_flag, block_id * rows_per_block, rows_per_block,
+                                           block_threads);
 }
 
 // ------------------------------------------------------------------------------------------------------------

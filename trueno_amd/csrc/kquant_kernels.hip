@@ -144,6 +144,47 @@ kq_gemv_group(u32 firsts0, u32 firsts1, u32 firsts2, u32 firsts3, u32 firsts4, u
   else if (e.fmt == FMT_Q6K) chain_step<FMT_Q6K, KQ_U>(e, nullptr, 0u, nullptr, lds4, &s_flag, block_id, num_blocks, block_threads);
 }
 
+// Any number of GEMVs that do not depend on one another in one launch of one workgroup per place on the chip: the
+// launcher cuts the entries' rows into items (entry, first row, rows) of equal cost per workgroup, in list order, so a
+// workgroup takes the end of one entry and the beginning of the next - or a slice of a large one - and all of them end
+// together; with many entries to a launch the fixed time of a launch (its first bytes arrive slowly, its last
+// workgroups run alone) is paid once for gigabytes.  Tables in device memory: wgs[2 b] = first item of workgroup b,
+// wgs[2 b + 1] = its number of items.  An item is computed exactly as a workgroup of a launch of its own would.
+struct GemvItem { u32 entry, row0, rows, pad; };
+// items i .. of this workgroup for as long as they are of format FMT (one loop per format: with the three engines side
+// by side in one loop body the register allocator needs half again as many registers)
+template <int FMT>
+__device__ __forceinline__ u32 many_run(u32 i, u32 count, const GemvItem* __restrict__ items, const GemvGroupHot* __restrict__ hot,
+                                        const GemvGroupCold* __restrict__ cold, f32x4* lds4, u32* s_flag, u32 block_threads) {
+  for (; i < count; ++i) {
+    const GemvItem it = items[i];
+    const GemvGroupHot h = hot[it.entry];
+    if (h.fmt != static_cast<u32>(FMT)) break;
+    const GemvGroupCold c = cold[it.entry];
+    const ChainEntry e = {h.fmt, h.k, h.n, h.flags, h.w, h.x, c.y, c.gamma, c.x2, c.residual, c.eps, 0u};
+    chain_step_rows<FMT, KQ_U>(e, nullptr, 0u, nullptr, lds4, s_flag, it.row0, it.rows, block_threads);
+    __syncthreads();      // the next item's vector goes where this one's partial sums are still being read
+  }
+  return i;
+}
+extern "C" __global__ void __launch_bounds__(768)
+kq_gemv_many(const u32* __restrict__ wgs, const GemvItem* __restrict__ items, const GemvGroupHot* __restrict__ hot,
+             const GemvGroupCold* __restrict__ cold) {
+  extern __shared__ f32x4 lds4[];
+  __shared__ u32 s_flag;
+  const u32 count = wgs[2u * blockIdx.x + 1u];
+  items += wgs[2u * blockIdx.x];
+  const u32 block_threads = blockDim.x;
+  u32 i = 0;
+  while (i < count) {
+    const u32 fmt = hot[items[i].entry].fmt;
+    if (fmt == FMT_Q4K) i = many_run<FMT_Q4K>(i, count, items, hot, cold, lds4, &s_flag, block_threads);
+    else if (fmt == FMT_Q5K) i = many_run<FMT_Q5K>(i, count, items, hot, cold, lds4, &s_flag, block_threads);
+    else if (fmt == FMT_Q6K) i = many_run<FMT_Q6K>(i, count, items, hot, cold, lds4, &s_flag, block_threads);
+    else ++i;
+  }
+}
+
 // The list as phases of independent entries in one resident launch, one workgroup of 12 waves per CU.
 extern "C" __global__ void __launch_bounds__(768)
 kq_gemv_phases(const ChainEntry* entries, const PhaseAssign* assign, u32 phases, u32* counters, u32* status, u32 spin_limit) {

@@ -18,6 +18,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -74,7 +75,7 @@ struct DeviceKernels {
   hipModule_t module = nullptr;
   int cu_count = 0;
   hipFunction_t gemv_fast[NFMT] = {}, gemv_flags[NFMT] = {}, gemv_generic[NFMT] = {};
-  hipFunction_t fill_u32 = nullptr, gemv_group = nullptr, phases = nullptr;
+  hipFunction_t fill_u32 = nullptr, gemv_group = nullptr, gemv_many = nullptr, phases = nullptr;
   int cooperative = 0;
   uint32_t resident_small = 3;   // resident 256-thread GEMV workgroups per CU (occupancy of the one-slab geometry)
   hipFunction_t gemm_fast[NFMT] = {}, gemm_generic[NFMT] = {}, gemm_as_written[NFMT] = {};
@@ -92,6 +93,7 @@ std::mutex g_mutex;
 // The tuning knobs are process-wide and meant for tests and measurements: atomics, so that a thread that flips one
 // while another launches is a race on the setting, never on memory.
 DeviceKernels g_dev[kMaxDevices];
+std::atomic<int> g_tune_epoch{0};           // counts the calls of trn_set_tuning: plans made under other settings are stale
 std::atomic<int> g_tune_blocks_per_cu{0};
 std::atomic<int> g_tune_row_groups{0};
 std::atomic<int> g_tune_batch_mode{0};   // 0: launches (default); 1: resident phases + barriers
@@ -110,6 +112,10 @@ std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds 
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
 std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4, 8 or (Q4_K) 12 (0: default)
 std::atomic<int> g_tune_stream_off{0};      // 1: one-slab GEMVs load their rows into registers straight from memory (no LDS ring)
+std::atomic<int> g_tune_stream_q6k{0};      // 1: Q6_K one-slab GEMVs stream through LDS too
+std::atomic<int> g_tune_stream_cost{0};     // percent of its bytes a streamed entry counts for when a grouped launch shares out its workgroups (0: default)
+std::atomic<int> g_tune_stream_min_rows{0}; // a single GEMV streams when a wave gets at least this many rows (0: default)
+std::atomic<int> g_tune_many_waves{0};      // waves per workgroup of a launch of more than sixteen entries (0: 12)
 std::atomic<int> g_tune_stream_waves{0};    // waves per workgroup of a single streamed GEMV (0: default)
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
@@ -162,6 +168,7 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.rmsnorm, "rmsnorm")) != hipSuccess ||
         (e = get_fn(m, &t.residual_rmsnorm, "fused_residual_rmsnorm")) != hipSuccess ||
         (e = get_fn(m, &t.gemv_group, "kq_gemv_group")) != hipSuccess ||
+        (e = get_fn(m, &t.gemv_many, "kq_gemv_many")) != hipSuccess ||
         (e = get_fn(m, &t.phases, "kq_gemv_phases")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_simplified, "q4k_gemm_fused")) != hipSuccess ||
         (e = get_fn(m, &t.dequant_simplified, "q4k_simplified_dequant_f32")) != hipSuccess ||
@@ -208,7 +215,12 @@ struct GemvGeometry {
 };
 
 // Can an n x k matrix of this format go through the streamed engine?  (one slab; any alignment the fast kernels take)
-bool stream_ok(uint32_t k) { return !g_tune_stream_off && k != 0 && k <= 4096u; }
+// Q6_K stays on the register path: its 210-byte blocks lie at 2-byte alignment in LDS too, and the five reads per row
+// that start there cost more than the whole-line copies gain (eight 4096 x 4096 per call 3.18 -> 3.38 us a matrix,
+// 32000 x 4096 19.4 -> 19.9 us; Q4_K 11008 x 4096 5.02 -> 4.53 us, Q5_K 6.57 -> 6.29 us).  "gemv_stream_q6k" turns it on.
+bool stream_ok(uint32_t fmt_code, uint32_t k) {
+  return !g_tune_stream_off && k != 0 && k <= 4096u && (fmt_code != 6u || g_tune_stream_q6k);
+}
 
 // Geometry of a single streamed GEMV: workgroups of `waves` waves, as many per CU as their LDS allows (two by default).
 GemvGeometry stream_geometry(const DeviceKernels& d, Fmt f, uint32_t k, uint32_t n) {
@@ -225,6 +237,10 @@ GemvGeometry stream_geometry(const DeviceKernels& d, Fmt f, uint32_t k, uint32_t
   rows = std::max<uint64_t>(ug, (rows + ug - 1) / ug * ug);
   const uint64_t max_rows = (kStreamLdsLimit - fixed) / 4u / ug * ug;
   rows = std::min<uint64_t>(rows, max_rows);
+  // A wave that gets only a batch or two never reaches the steady state the ring is there for, and the start of a
+  // streamed workgroup is the longer one (Q4_K 4096 x 4096 alone: 5.2 us on the register path, 6.4 us streamed).
+  const uint32_t min_rows = g_tune_stream_min_rows > 0 ? uint32_t(g_tune_stream_min_rows) : 16u;
+  if (rows < uint64_t(min_rows) * waves) return g;
   g.grid = uint32_t((uint64_t(n) + rows - 1) / rows);
   g.block = 64u * waves;
   g.lds = uint32_t(fixed + rows * 4u);
@@ -557,7 +573,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void* gemm_args[] = {&a, &w, &c, &m, &n, &k};
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
-  if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(k)) {
+  if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(uint32_t(f) + 4u, k)) {
     g = stream_geometry(*d, f, k, n);
     if (g.fits) {
       flags |= kChainStreamFlag;
@@ -687,39 +703,54 @@ uint32_t chain_barrier_stride_host(uint32_t num_workgroups) { return 64u * (1u +
 constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (kGroupEntries of the kernel)
 // what a further slab of 4096 columns adds to the cost of an entry's bytes when workgroups are shared out (launch_gemv_group)
 constexpr double kSlabCost = 0.4;
+// what a streamed entry's bytes cost against an entry's on the register path (launch_gemv_group)
+constexpr double kStreamCost = 0.95;
 // Entries a launch takes by default: as many as the kernel holds, looked for among the next 32 of the list.  On the 7B
 // pass with activation buffers per layer: 8 entries (138 MB a launch, 30 launches) 879 us, 12 of the next 24 (21
 // launches) 820 us, 14 of 28 (18) 821 us, 16 of 32 (16 launches of 270 MB) 823 us; the launches of 12-16 entries run at
 // 4.8-5.4 TB/s against 4.3-4.7 for 8.  (Before the workgroups of a launch were kept within the number resident at once -
 // launch_gemv_group - sixteen entries measured 1075 us: shares rounded up to 260 workgroups for 256 places.)
 constexpr uint32_t kGroupDefault = 16;
+// Beyond kGroupMax entries a launch takes its entries from tables in device memory (launch_gemv_many): as many mutually
+// independent entries as the list offers, looked for over the whole list.  The 7B pass with activation buffers per layer
+// is then three launches - the 160 q, k, v, gate and up matrices (2.5 GB), the 64 o and down matrices (1.5 GB), the head -
+// where sixteen entries a launch made 16 launches of 258 MB, each paying 5-7 us of fixed time over a bare read.
+constexpr uint32_t kManyMax = 4096;
 bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d) {
   return d.n != 0 && d.k != 0 && d.x && d.w && d.y && gemv_fast_ok(Fmt(d.fmt - 4), d.y, d.w, d.x) &&
          gemv_geometry(*dk, d.k, d.n).fits;
 }
 
-// Cuts a list into launches (mode 0).  A launch is filled with up to kGroupMax entries that are independent of one
+// Cuts a list into launches (mode 0).  A launch is filled with up to group_max entries that are independent of one
 // another AND of every earlier entry that has not been launched yet: the first entry still waiting always goes in,
 // later ones of a window are brought forward when nothing they read or write is touched by an entry they would
 // overtake.  What an entry computes does not depend on the company it is launched in, so the results are those of
-// the list in order.
-void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches) {
-  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : 2u * kGroupDefault);
-  const uint32_t group_max =
-      g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), kGroupMax) : kGroupDefault);
-  std::vector<uint8_t> launched(count, 0);
+// the list in order.  many_ok: launches of more than kGroupMax entries may be made (not while the stream is being
+// captured into a graph: their tables are uploaded by a copy).
+void schedule_list(DeviceKernels* dk, const trn_gemv_desc* descs, uint32_t count, std::vector<std::vector<uint32_t>>* launches,
+                   bool many_ok = true) {
+  const uint32_t cap = many_ok ? kManyMax : kGroupMax;
+  const uint32_t group_max = g_tune_group_off ? 1u : (g_tune_group_max > 0 ? std::min<uint32_t>(uint32_t(g_tune_group_max), cap) : cap);
+  const uint32_t window = g_tune_group_off ? 1u : (g_tune_group_window > 0 ? uint32_t(g_tune_group_window) : std::max(2u * kGroupDefault, 2u * group_max));
+  std::vector<uint8_t> launched(count, 0), groupable(count, 0);
+  for (uint32_t i = 0; i < count; ++i) groupable[i] = list_groupable(dk, descs[i]) ? 1 : 0;
+  // conflicts between an entry and the (at most window - 1) entries before it, looked up many times below
+  const uint32_t span = std::min(window, count);
+  std::vector<uint8_t> conf(size_t(count) * span, 0);      // conf[j * span + (j - i)] for 0 < j - i < span
+  for (uint32_t j = 0; j < count; ++j)
+    for (uint32_t i = j > span - 1 ? j - (span - 1) : 0; i < j; ++i)
+      conf[size_t(j) * span + (j - i)] = (desc_conflict(descs[j], descs[i]) || desc_conflict(descs[i], descs[j])) ? 1 : 0;
   for (uint32_t pos = 0; pos < count;) {
     if (launched[pos]) { ++pos; continue; }
     std::vector<uint32_t> members(1, pos);
-    if (list_groupable(dk, descs[pos])) {
+    if (groupable[pos]) {
       const uint32_t end = uint32_t(std::min<uint64_t>(count, uint64_t(pos) + window));
       for (uint32_t j = pos + 1; j < end && members.size() < group_max; ++j) {
         if (launched[j]) continue;
-        const trn_gemv_desc& c = descs[j];
-        if (!list_groupable(dk, c)) break;           // an entry that takes another path keeps its place in the order
+        if (!groupable[j]) break;                    // an entry that takes another path keeps its place in the order
         bool ok = true;
         for (uint32_t i = pos; i < j && ok; ++i)     // the members of the launch and everything it would overtake
-          if (!launched[i]) ok = !desc_conflict(c, descs[i]) && !desc_conflict(descs[i], c);
+          if (!launched[i]) ok = !conf[size_t(j) * span + (j - i)];
         if (ok) members.push_back(j);
       }
     }
@@ -1163,6 +1194,9 @@ trn_status trn_stream_create(trn_stream* stream, unsigned flags) {
   return TRN_SUCCESS;
 }
 
+namespace {
+void release_list_plans(hipStream_t stream);      // the cached plans of trn_kquant_gemv_batch and their device tables (defined with them)
+}
 // The per-(device, stream) scratch buffers of a stream that is going away (partial sums, arrival counters, the
 // resident executor's tables).  The stream must be idle.
 static void release_stream_workspaces(hipStream_t stream) {
@@ -1180,6 +1214,7 @@ static void release_stream_workspaces(hipStream_t stream) {
   drop_simple(g_gemv_f32_ws);
   drop_simple(g_attention_ws);
   drop_simple(g_gemm_ws);
+  release_list_plans(stream);
   for (auto it = g_chain_ws.begin(); it != g_chain_ws.end();) {
     if (it->first.second == stream) {
       ChainWorkspace& w = it->second;
@@ -1355,7 +1390,11 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   auto cost_of = [&](const trn_gemv_desc& e) {
     const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
     const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
-    return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
+    // a streamed entry's bytes arrive faster than those of an entry on the register path
+    const bool streamed = stream_ok(e.fmt, e.k) &&
+                          uint64_t(e.k) * 4u + kLdsScratch + waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) + kGemvRowsPerBatch * 4u <= kStreamLdsLimit;
+    const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
+    return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u)) * (streamed ? stream_cost : 1.0);
   };
   for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
   // the kernels hold 3 waves per SIMD, 12 per CU
@@ -1368,7 +1407,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   // an entry of one slab streams its rows through LDS when the rings of all waves fit beside its vector
   auto ring_of = [&](uint32_t i) -> uint32_t {
     const trn_gemv_desc& e = descs[i];
-    if (!stream_ok(e.k)) return 0u;
+    if (!stream_ok(e.fmt, e.k)) return 0u;
     const uint32_t ring = waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]);
     return uint64_t(e.k) * 4u + kLdsScratch + ring + kGemvRowsPerBatch * 4u <= kStreamLdsLimit ? ring : 0u;
   };
@@ -1449,6 +1488,134 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   for (uint32_t a = 0; a < 8; ++a) packed[a] = first[2 * a + 1] | first[2 * a + 2] << 16;
   void* args[] = {&packed[0], &packed[1], &packed[2], &packed[3], &packed[4], &packed[5], &packed[6], &packed[7], &g};
   return hipModuleLaunchKernel(d->gemv_group, first[len], 1, 1, 64u * waves, 1, 1, lds, stream, args, nullptr);
+}
+
+// ---- launches of more than kGroupMax entries: tables in device memory (kq_gemv_many) ------------------------------
+struct ManyTables {
+  std::vector<uint32_t> host;     // [2 per workgroup: first item, items][4 per item: entry, row0, rows, 0][Hot per entry][Cold per entry]
+  void* dev = nullptr;
+  uint32_t grid = 0, block = 0, lds = 0;
+  size_t off_items = 0, off_hot = 0, off_cold = 0;     // in bytes
+};
+
+// Cuts the rows of len mutually independent entries (all meeting the fast kernels' preconditions) into items for one
+// workgroup per place on the chip: the entries lie one behind the other on an axis of cost (bytes, weighted as in
+// launch_gemv_group), the axis is cut into equal parts, and a workgroup's items are the pieces of entries inside its
+// part - whole batches of rows; a piece of fewer than 32 rows at either end of an entry goes to the neighbour, and an
+// item holds no more rows than its partial sums have room for in LDS.
+hipError_t plan_gemv_many(DeviceKernels* d, const trn_gemv_desc* descs, uint32_t len, ManyTables* t) {
+  // twelve waves to a workgroup, one workgroup per CU (the 7B pass: 764 us with eight, 752 us with twelve; the short
+  // launches of launch_gemv_group are the other way round)
+  uint32_t waves = g_tune_many_waves > 0 ? std::min(uint32_t(g_tune_many_waves), kGemvMaxWaves) : kGemvMaxWaves;
+  for (uint32_t i = 0; i < len; ++i) {
+    const GemvGeometry alone = gemv_geometry(*d, descs[i].k, descs[i].n);
+    if (!alone.fits) return hipErrorInvalidValue;
+    waves = std::max(waves, alone.block / 64u);
+  }
+  const uint32_t G = uint32_t(d->cu_count) * (g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::max(1u, 12u / waves));
+  const uint32_t ug = kGemvRowsPerBatch;
+  struct Ent { double cost; uint32_t ring, sw, max_rows; uint64_t x_bytes; };
+  std::vector<Ent> ent(len);
+  double total = 0.0;
+  for (uint32_t i = 0; i < len; ++i) {
+    const trn_gemv_desc& e = descs[i];
+    const uint32_t slabs = (e.k / 256u + 15u) / 16u, sw = std::min(slabs, waves);
+    uint32_t ring = stream_ok(e.fmt, e.k) ? waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) : 0u;
+    const uint64_t x_bytes = uint64_t(e.k) * 4u;
+    if (ring && x_bytes + kLdsScratch + ring + ug * 4u > kStreamLdsLimit) ring = 0u;
+    const uint64_t limit = ring ? kStreamLdsLimit - ring : kFastLdsLimit;
+    if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > limit) return hipErrorInvalidValue;
+    const uint32_t max_rows = uint32_t(std::min<uint64_t>((limit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug, 1u << 20));
+    const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
+    const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
+    const double cost = double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (sw - 1u)) * (ring ? stream_cost : 1.0);
+    ent[i] = {cost, ring, sw, max_rows, x_bytes};
+    total += cost;
+  }
+  const double part = total / G;
+  std::vector<std::vector<uint32_t>> items_of(G);      // per workgroup: (entry, row0, rows) triples
+  uint32_t lds = 0;
+  double start = 0.0;
+  for (uint32_t i = 0; i < len; ++i) {
+    const trn_gemv_desc& e = descs[i];
+    const double end = start + ent[i].cost;
+    const uint32_t w0 = std::min(G - 1u, uint32_t(start / part)), w1 = std::min(G - 1u, uint32_t(std::max(start, end - 1e-9 * part) / part));
+    uint32_t row = 0;
+    for (uint32_t w = w0; w <= w1 && row < e.n; ++w) {
+      uint32_t upto = e.n;
+      if (w < w1) {
+        const double frac = (double(w + 1u) * part - start) / ent[i].cost;
+        upto = uint32_t(std::min<double>(double(e.n), std::max(0.0, frac * double(e.n)) + 0.5)) / ug * ug;
+        if (upto < row + 32u) continue;                 // too small a piece at the entry's start: the next workgroup takes it
+        if (e.n - upto < 32u) upto = e.n;               // ... at its end: this one takes it
+      }
+      while (row < upto) {
+        const uint32_t rows = std::min((upto - row + ug - 1u) / ug * ug, ent[i].max_rows);
+        items_of[w].insert(items_of[w].end(), {i, row, rows});
+        lds = std::max<uint32_t>(lds, uint32_t(ent[i].x_bytes + uint64_t(ent[i].sw) * rows * 4u + kLdsScratch + ent[i].ring));
+        row += rows;
+      }
+    }
+    start = end;
+  }
+  size_t n_items = 0;
+  for (const auto& v : items_of) n_items += v.size() / 3u;
+  const size_t words = 2u * size_t(G) + 4u * n_items + 20u * size_t(len);
+  t->host.assign(words, 0u);
+  t->off_items = 8u * size_t(G);
+  t->off_hot = t->off_items + 16u * n_items;
+  t->off_cold = t->off_hot + 40u * size_t(len);
+  uint32_t next = 0;
+  for (uint32_t w = 0; w < G; ++w) {
+    t->host[2u * w] = next;
+    t->host[2u * w + 1u] = uint32_t(items_of[w].size() / 3u);
+    for (size_t k = 0; k < items_of[w].size(); k += 3, ++next) {
+      uint32_t* it = &t->host[t->off_items / 4u + 4u * next];
+      it[0] = items_of[w][k]; it[1] = items_of[w][k + 1]; it[2] = items_of[w][k + 2];
+    }
+  }
+  for (uint32_t i = 0; i < len; ++i) {
+    const trn_gemv_desc& e = descs[i];
+    const GemvGroupHost::Hot hot = {e.w, e.x, e.k, e.n, e.fmt, e.flags | (ent[i].ring ? kChainStreamFlag : 0u), 0u, 0u};
+    const GemvGroupHost::Cold cold = {e.y, e.gamma, e.x2, e.residual, e.norm_eps, 0u};
+    std::memcpy(reinterpret_cast<uint8_t*>(t->host.data()) + t->off_hot + 40u * i, &hot, 40);
+    std::memcpy(reinterpret_cast<uint8_t*>(t->host.data()) + t->off_cold + 40u * i, &cold, 40);
+  }
+  t->grid = G;
+  t->block = 64u * waves;
+  t->lds = lds;
+  return hipSuccess;
+}
+
+// What trn_kquant_gemv_batch does with a list, kept per (device, stream) for as long as the same list comes again (a
+// decoder issues the same list for every token): the cut into launches and the device tables of the large launches.
+struct PlannedLaunch {
+  std::vector<uint32_t> members;
+  ManyTables many;             // used when the launch has more than kGroupMax entries
+};
+struct ListPlan {
+  std::vector<trn_gemv_desc> key;
+  int epoch = -1;
+  std::vector<PlannedLaunch> launches;
+};
+std::map<std::tuple<int, hipStream_t, bool>, ListPlan> g_list_plans;     // by device, stream and "may make large launches"; under g_ws_mutex
+
+void free_plan_tables(ListPlan* plan) {
+  for (PlannedLaunch& l : plan->launches)
+    if (l.many.dev) {
+      (void)hipFree(l.many.dev);
+      l.many.dev = nullptr;
+    }
+}
+void release_list_plans(hipStream_t stream) {       // under g_ws_mutex; the stream is idle
+  for (auto it = g_list_plans.begin(); it != g_list_plans.end();) {
+    if (std::get<1>(it->first) == stream) {
+      free_plan_tables(&it->second);
+      it = g_list_plans.erase(it);
+    } else {
+      ++it;
+    }
+  }
 }
 }  // namespace
 
@@ -1535,15 +1702,64 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   bool handled = false;
   e = launch_chain(stream, descs, count, &handled);
   if (handled || e != hipSuccess) return st(e);
-  std::vector<std::vector<uint32_t>> launches;
-  schedule_list(dk, descs, count, &launches);
+  int dev = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return st(e);
+  // while the stream is being captured into a graph nothing may be copied or allocated: kernel-argument launches only
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    capturing = hipStreamCaptureStatusNone;
+  }
+  const bool many_ok = capturing == hipStreamCaptureStatusNone;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  ListPlan& plan = g_list_plans[std::make_tuple(dev, stream, many_ok)];      // (a capture has a plan of its own)
+  const bool same = plan.epoch == g_tune_epoch && plan.key.size() == count &&
+                    std::memcmp(plan.key.data(), descs, size_t(count) * sizeof(trn_gemv_desc)) == 0;
+  if (!same) {
+    bool had_tables = false;
+    for (const PlannedLaunch& l : plan.launches) had_tables = had_tables || l.many.dev;
+    if (had_tables) {      // (never during a capture: its plans have no tables)
+      if ((e = hipStreamSynchronize(stream)) != hipSuccess) return st(e);   // a launch in flight may still read the old tables
+      free_plan_tables(&plan);
+    }
+    plan.launches.clear();
+    plan.key.assign(descs, descs + count);
+    plan.epoch = g_tune_epoch;
+    std::vector<std::vector<uint32_t>> cut;
+    schedule_list(dk, descs, count, &cut, many_ok);
+    std::vector<trn_gemv_desc> group;
+    for (std::vector<uint32_t>& members : cut) {
+      PlannedLaunch pl;
+      pl.members = std::move(members);
+      if (pl.members.size() > kGroupMax) {
+        group.clear();
+        for (uint32_t m : pl.members) group.push_back(descs[m]);
+        if ((e = plan_gemv_many(dk, group.data(), uint32_t(group.size()), &pl.many)) != hipSuccess ||
+            (e = hipMalloc(&pl.many.dev, pl.many.host.size() * 4u)) != hipSuccess ||
+            (e = hipMemcpy(pl.many.dev, pl.many.host.data(), pl.many.host.size() * 4u, hipMemcpyHostToDevice)) != hipSuccess) {
+          if (pl.many.dev) (void)hipFree(pl.many.dev);
+          free_plan_tables(&plan);
+          plan.launches.clear();
+          plan.key.clear();
+          return st(e);
+        }
+      }
+      plan.launches.push_back(std::move(pl));
+    }
+  }
   std::vector<trn_gemv_desc> group;
-  for (const std::vector<uint32_t>& members : launches) {
+  for (const PlannedLaunch& pl : plan.launches) {
+    const std::vector<uint32_t>& members = pl.members;
     const trn_gemv_desc& head = descs[members[0]];
     // a large matrix alone (the 108 MB head of the 7B pass) is 2-4 us faster as a group of one: workgroups of 8 waves that
     // hand their rows out among themselves; smaller ones alone (37 MB, 9 MB) are slower that way
     const bool big_single = list_groupable(dk, head) && double(head.n) * (head.k / 256u) * kSbBytes[head.fmt - 4] >= 64e6;
-    if (members.size() >= 2 || big_single || (desc_extended(head) && list_groupable(dk, head))) {
+    if (pl.many.dev) {
+      uint64_t wgs = reinterpret_cast<uint64_t>(pl.many.dev), items = wgs + pl.many.off_items, hot = wgs + pl.many.off_hot,
+               cold = wgs + pl.many.off_cold;
+      void* args[] = {&wgs, &items, &hot, &cold};
+      e = hipModuleLaunchKernel(dk->gemv_many, pl.many.grid, 1, 1, pl.many.block, 1, 1, pl.many.lds, stream, args, nullptr);
+    } else if (members.size() >= 2 || big_single || (desc_extended(head) && list_groupable(dk, head))) {
       group.clear();
       for (uint32_t m : members) group.push_back(descs[m]);
       e = launch_gemv_group(dk, stream, group.data(), uint32_t(group.size()));
@@ -1670,6 +1886,7 @@ trn_status trn_device_cu_count(int* count) {
 trn_status trn_set_tuning(const char* key, int value) {
   if (!key || value < 0) return TRN_ERROR_INVALID_VALUE;
   std::lock_guard<std::mutex> lock(g_mutex);
+  ++g_tune_epoch;
   if (!std::strcmp(key, "gemv_blocks_per_cu")) { g_tune_blocks_per_cu = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_row_groups")) { g_tune_row_groups = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "batch_mode")) {
@@ -1691,6 +1908,10 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "attention_min_steps")) { g_tune_attention_min_steps = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_off")) { g_tune_stream_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_waves")) { g_tune_stream_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "many_waves")) { g_tune_many_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemv_stream_q6k")) { g_tune_stream_q6k = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemv_stream_cost")) { g_tune_stream_cost = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemv_stream_min_rows")) { g_tune_stream_min_rows = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
