@@ -16,13 +16,18 @@ last layer's outputs and the logits are checked against fp64 on their actual inp
 GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate;
 h <- down) are timed too: `strict_decoder_chain` in `config`.
 
-Prints one JSON line.  `roofline`: the dominant kernel (kq_gemv_group: the launches that carry several
-independent entries and the head alone: the 16 launches of a pass), those launches timed with HIP events on their stream
-over as many rounds as the headline has passes, with the time of a bare read of as many bytes beside it; `cpu_baseline`: the CPU port
-(oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other
-benchmark configurations, timed as launches back to back over at least 1 GiB of distinct copies
-(200 launches, median of 5 batches), one copy over and over ("hot": from the last-level cache), and
-eight independent copies per library call (the grouped launch in steady state).
+Prints one JSON line.  `per_pass_us` (in `extra`): minimum, median and maximum of the K timed passes, from one HIP event
+between consecutive passes of the timed region itself.  `roofline`: the dominant kernel, kq_gemv_many (the two launches
+of a pass that take their many entries from tables in device memory: the 160 q, k, v, gate, up matrices, then the 64 o and
+down matrices; the head alone runs kq_gemv_group).  Its launches are timed with HIP events on their stream in a second
+region of the same K passes after the same W warm-up passes, each pass issued as its launches one list each with an event
+between them; that region's time per pass is reported beside the headline's.  `bare_read_*`: a launch that only reads as
+many bytes (non-temporal 16-byte loads, whole lines once), same protocol.  `cpu_baseline`: the CPU port
+(oracle/cpu_baseline.cpp) on layer 0's seven matrices with all host cores.  `extra` holds the other benchmark
+configurations, timed as launches back to back over at least 1 GiB of distinct copies (200 launches, median of 5
+batches), one copy over and over ("hot": from the last-level cache), and eight independent copies per library call (the
+grouped launch in steady state).  A 4 KB read (kq_read_u128 with one workgroup) is launched just outside each of the two
+regions: in a kernel trace it marks where they begin and end (rocprof_summary.py timed).
 """
 import argparse
 import ctypes as C
@@ -40,8 +45,8 @@ HBM_PEAK_GBPS = 8000.0
 TOL = 1e-5                      # relative L2 against fp64, as in the parity tests
 GIB = 1 << 30
 # HBM bytes per kq_gemv_group launch as the hardware counters saw them: written next to the rocprofv3 summaries by
-# the script that makes them (python -m trueno_amd.rocprof_summary), with the commit it was measured at.
-TRAFFIC_JSON = os.path.join(ROOT, "profiles", "kquant_gemv_group_traffic.json")
+# the script that makes them (python rocprof_summary.py), with the commit it was measured at.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "kquant_gemv_many_traffic.json")
 
 
 def main() -> int:
@@ -51,13 +56,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10, help="untimed passes first (the clocks take some ten milliseconds of load to settle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the tables of configurations 1, 2, 3 and 5 and of the path's neighbours")
-    ap.add_argument("--no-executors", action="store_true", help="skip the comparison run of the opt-in one-launch executor")
+    ap.add_argument("--executors", action="store_true", help="also time the opt-in one-launch executor (batch_mode 1; slower than launches on every list)")
     ap.add_argument("--pass-only", action="store_true",
                     help="only the timed passes and the launches of the roofline figure (for counter runs: every dispatch of the "
                          "dominant kernel then belongs to the pass)")
     args = ap.parse_args()
     if args.pass_only:
-        args.no_cpu_baseline = args.no_configs = args.no_executors = True
+        args.no_cpu_baseline = args.no_configs = True
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus must be 1 (several GPUs would each take a range of rows of "
               "every matrix and exchange the output vectors)", file=sys.stderr)
@@ -121,22 +126,42 @@ def main() -> int:
         assert L.trn_event_elapsed_ms(C.byref(ms), a, b) == 0
         return float(ms.value)
 
-    def run_passes(steps, warmup, batch=batch):
+    mark = t.GpuBuffer(ctx, 2048, np.float32)
+
+    def region_mark():
+        # a 4 KB read: in a kernel trace it separates what follows from what came before
+        L.trn_read_u128(stream.raw(), mark.as_ptr(), 4096, mark.as_ptr() + 4096)
+
+    pass_events = [ev() for _ in range(args.steps + 1)]
+
+    def run_passes(steps, warmup, batch=batch, events=None, marks=False):
+        """W untimed passes, then exactly K: wall clock per pass between two synchronisations, and the device's own time per
+        pass between the events around the K passes.  events: K + 1 events, one recorded between consecutive passes."""
         for _ in range(warmup):
             batch.launch(stream)
+        if marks:
+            region_mark()
         stream.synchronize()
         t0 = time.perf_counter()
-        L.trn_event_record(e0, stream.raw())
-        for _ in range(steps):
+        L.trn_event_record(events[0] if events else e0, stream.raw())
+        for i in range(steps):
             batch.launch(stream)
-        L.trn_event_record(e1, stream.raw())
+            if events and i + 1 < steps:
+                L.trn_event_record(events[i + 1], stream.raw())
+        L.trn_event_record(events[steps] if events else e1, stream.raw())
         stream.synchronize()
         wall = (time.perf_counter() - t0) * 1e3
-        return wall / steps, elapsed_ms(e0, e1) / steps
+        if marks:
+            region_mark()
+            stream.synchronize()
+        first, last = (events[0], events[steps]) if events else (e0, e1)
+        return wall / steps, elapsed_ms(first, last) / steps
 
     # ---- timed region: W warm-up passes, then exactly K passes ------------------------------------------------
-    ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup)
+    ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup, events=pass_events, marks=True)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
+    per_pass = sorted(elapsed_ms(pass_events[i], pass_events[i + 1]) * 1e3 for i in range(args.steps))
+    per_pass_us = {"min": round(per_pass[0], 1), "median": round(per_pass[len(per_pass) // 2], 1), "max": round(per_pass[-1], 1)}
 
     # ---- what the timed passes left behind, against fp64 on the actual inputs: the last layer and the logits ------
     def norm64(v, eps=1e-6):
@@ -157,60 +182,62 @@ def main() -> int:
     assert np.all(np.isfinite(got["logits"])) and worst <= TOL, f"the timed pass is wrong: {verification}"
     del host_last, host_head
 
-    # ---- dominant kernel: kq_gemv_group.  The library puts entries that are independent of one another (and of what
-    #      they would overtake) into one launch of this kernel; trn_kquant_gemv_plan says which entry of the pass goes
-    #      into which launch.  A launch of two or more entries runs this kernel, and so does a single matrix of 64 MB or
-    #      more (the head): on this pass that is every launch.  They are issued here one list each, in pass order, back
-    #      to back on the stream, bracketed by HIP events on that stream.
+    # ---- dominant kernel: kq_gemv_many.  The library puts entries that are independent of one another (and of what
+    #      they would overtake) into one launch; trn_kquant_gemv_plan says which entry of the pass goes into which.  A
+    #      launch of more than sixteen entries runs kq_gemv_many: on this pass the first two launches, 97 % of the bytes.
+    #      Second region: the same W + K passes, each pass issued as its launches one list each, in order, with an event
+    #      between them on the stream.
     launch_of = batch.plan()
     members = {}
     for i, l in enumerate(launch_of):
         members.setdefault(l, []).append(i)
-    kinds = {}
+    lists, dominant = [], []
     for l in sorted(members):
-        sig = "[" + ",".join(entry_names[i] for i in members[l]) + "] " + f"{sum(entry_bytes[i] for i in members[l]) / 1e6:.1f} MB"
-        kinds[sig] = kinds.get(sig, 0) + 1
-    print("[bench] launches of the pass: " + ", ".join(f"{c} x {sig}" for sig, c in kinds.items()), file=sys.stderr, flush=True)
-    groups, grp_bytes = [], 0
-    for l in sorted(members):
-        if len(members[l]) >= 2 or entry_bytes[members[l][0]] >= 64e6 + 4 * (32000 + 4096):
-            g = batch.subset(members[l])
-            assert len(set(g.plan())) == 1, "a launch of the pass, issued alone, must again be one launch"
-            groups.append(g)
-            grp_bytes += sum(entry_bytes[i] for i in members[l])
-    n_grp = len(groups)
-    # as many rounds of these launches between the two events as the headline has passes (the clocks of a memory-bound
-    # run wander by several percent over milliseconds: one round alone read 55-66 us per launch on one box), three such
-    # measurements, the median
-    grp_ms = []
-    for _ in range(3):
-        for g in groups:
+        names = [entry_names[i] for i in members[l]]
+        kinds = sorted(set(names), key=names.index)
+        nbytes = sum(entry_bytes[i] for i in members[l])
+        print(f"[bench] launch {l}: {len(names)} entries ({', '.join(f'{names.count(k)} x {k}' for k in kinds)}), {nbytes / 1e6:.1f} MB",
+              file=sys.stderr, flush=True)
+        g = batch.subset(members[l])
+        assert len(set(g.plan())) == 1, "a launch of the pass, issued alone, must again be one launch"
+        lists.append((g, nbytes, len(names) > 16))
+    n_dom = sum(1 for _, _, dom in lists if dom)
+    assert n_dom >= 1, "the pass has no launch of more than sixteen entries: the roofline section needs rewriting"
+    dom_bytes = sum(nb for _, nb, dom in lists if dom)
+    evs = [[ev() for _ in range(len(lists) + 1)] for _ in range(args.steps)]
+    for _ in range(args.warmup):
+        for g, _, _ in lists:
             g.launch(stream)
-        stream.synchronize()
-        L.trn_event_record(e0, stream.raw())
-        for _ in range(args.steps):
-            for g in groups:
-                g.launch(stream)
-        L.trn_event_record(e1, stream.raw())
-        stream.synchronize()
-        grp_ms.append(elapsed_ms(e0, e1) / (n_grp * args.steps))
-    grp_ms = sorted(grp_ms)[len(grp_ms) // 2]
-    grp_bytes_per_launch = grp_bytes / n_grp
+    region_mark()
+    stream.synchronize()
+    for p in range(args.steps):
+        L.trn_event_record(evs[p][0], stream.raw())
+        for j, (g, _, _) in enumerate(lists):
+            g.launch(stream)
+            L.trn_event_record(evs[p][j + 1], stream.raw())
+    stream.synchronize()
+    region_mark()
+    stream.synchronize()
+    dom_us = sum(elapsed_ms(evs[p][j], evs[p][j + 1]) * 1e3 for p in range(args.steps) for j, (_, _, dom) in enumerate(lists) if dom)
+    grp_ms = dom_us / (n_dom * args.steps) * 1e-3
+    region2_us_per_pass = elapsed_ms(evs[0][0], evs[-1][-1]) * 1e3 / args.steps
+    per_launch_us = [round(sum(elapsed_ms(evs[p][j], evs[p][j + 1]) for p in range(args.steps)) * 1e3 / args.steps, 2) for j in range(len(lists))]
+    n_grp = n_dom
+    grp_bytes_per_launch = dom_bytes / n_dom
     achieved = grp_bytes_per_launch / (grp_ms * 1e-3) / 1e9
 
-    # a bare read of as many bytes per launch, nothing computed, launches back to back over cold data: what the
-    # memory system and a kernel launch allow for a launch of this size
+    # a bare read of as many bytes per launch, nothing computed (non-temporal 16-byte loads, every line once), launches
+    # back to back over cold data: what the memory system and a kernel launch allow for a launch of this size
     read_bytes = int(grp_bytes_per_launch) // 16 * 16
-    pieces = GIB // read_bytes
-    read_src = t.GpuBuffer(ctx, GIB // 4, np.float32)
+    read_src = t.GpuBuffer(ctx, (2 * read_bytes + 4) // 4, np.float32)
     read_us = []
     for _ in range(5):
         L.trn_event_record(e0, stream.raw())
-        for r in range(64):
-            L.trn_read_u128(stream.raw(), read_src.as_ptr() + (r % pieces) * read_bytes, read_bytes, y[4096].as_ptr())
+        for r in range(8):
+            L.trn_read_u128(stream.raw(), read_src.as_ptr() + (r % 2) * read_bytes, read_bytes, y[4096].as_ptr())
         L.trn_event_record(e1, stream.raw())
         stream.synchronize()
-        read_us.append(elapsed_ms(e0, e1) * 1e3 / 64)
+        read_us.append(elapsed_ms(e0, e1) * 1e3 / 8)
     read_us = sorted(read_us)[2]
     read_src.free()
 
@@ -237,7 +264,7 @@ def main() -> int:
 
     # ---- the same list through the one-launch executor (opt-in), for comparison ------------------------
     other_modes = {}
-    if not args.no_executors:
+    if args.executors:
         L.trn_set_tuning(b"batch_mode", 1)
         ms, _ = run_passes(max(3, args.steps // 2), 1)
         other_modes["resident_phases"] = round(ms * 1e3, 1)
@@ -247,8 +274,6 @@ def main() -> int:
     #      20 to warm up, then 5 batches of 200, the median batch counts.  "cold": every launch another of enough
     #      distinct device copies to make 1 GiB (nothing comes from the 256 MB last-level cache); "hot": one copy over
     #      and over; "grouped": eight copies per library call, which the library issues as one launch.
-    mark = t.GpuBuffer(ctx, 2048, np.float32)
-
     def protocol(launch, reps=200, warm=20, batches=5):
         # a 4 KB read in front: in a kernel trace it separates this configuration's launches from the last one's
         L.trn_read_u128(stream.raw(), mark.as_ptr(), 4096, mark.as_ptr() + 4096)
@@ -508,14 +533,18 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic["bytes_per_launch"] if traffic else None,
                      "traffic_measured_at": traffic.get("commit") if traffic else None,
-                     "kernel": "kq_gemv_group", "launches_per_pass": n_grp,
+                     "kernel": "kq_gemv_many", "launches_per_pass": n_grp,
                      "bytes_per_launch": round(grp_bytes_per_launch), "us_per_launch": round(grp_ms * 1e3, 3),
+                     # the region these launches were timed in: every launch of a pass as a list of its own, events between
+                     "us_per_pass_in_this_region": round(region2_us_per_pass, 1), "us_per_launch_of_the_pass_in_order": per_launch_us,
+                     # the whole pass of the headline region against the peak (head, launch gaps and all): a lower bound
+                     "frac_of_peak_from_ms_per_step": round(value / HBM_PEAK_GBPS, 4),
                      # a launch that only reads as many bytes (trn_read_u128), same protocol: the ceiling for a launch of this size
                      "bare_read_us_per_launch": round(read_us, 3), "bare_read_gbps": round(read_bytes / read_us / 1e3, 1),
                      "frac_of_bare_read": round(read_us / (grp_ms * 1e3), 4)},
         "cpu_baseline": cpu,
         "extra": {"us_per_pass": round(ms_per_step * 1e3, 1), "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-                  "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1),
+                  "gpu_event_us_per_pass": round(gpu_ms_per_step * 1e3, 1), "per_pass_us": per_pass_us,
                   "verification_after_timed_region_rel_l2_vs_fp64": dict(verification, tolerance=TOL),
                   "us_per_pass_strict_decoder_chain": strict_ms and round(strict_ms * 1e3, 1),
                   "us_per_pass_one_launch_executors": other_modes,

@@ -1,22 +1,26 @@
 """Summaries of rocprofv3 runs of bench.py, from the rocpd SQLite files rocprofv3 writes (`*_results.db`).
 
-  python -m trueno_amd.rocprof_summary trace <dir>
+  python rocprof_summary.py trace <dir>
       per kernel and launch shape: calls, average / min / max duration in microseconds (a Markdown table)
-  python -m trueno_amd.rocprof_summary traffic <fetch_dir> <write_dir> [--kernel kq_gemv_group] [--json out.json]
+  python rocprof_summary.py traffic <fetch_dir> <write_dir> [--kernel kq_gemv_many] [--json out.json]
       HBM bytes per launch of one kernel from two counter runs (`--pmc FETCH_SIZE`, `--pmc WRITE_SIZE`, KiB per
       dispatch), each scaled by what the same counter reads for the 256 MiB kq_copy_u128 of the same run; with --json the
       figure bench.py reports as `roofline.traffic` is written, stamped with the commit of the working tree.
-  python -m trueno_amd.rocprof_summary shapes <fetch_dir> <write_dir> [--prefix q4k_gemm]
+  python rocprof_summary.py shapes <fetch_dir> <write_dir> [--prefix q4k_gemm]
       the same two counters per kernel and launch shape (a Markdown table): for kernels that serve several shapes
-  python -m trueno_amd.rocprof_summary runs <trace_dir> [<fetch_dir> <write_dir>] [--prefix q4k_gemm] [--min 100]
+  python rocprof_summary.py runs <trace_dir> [<fetch_dir> <write_dir>] [--prefix q4k_gemm] [--min 100]
       runs of consecutive dispatches of one kernel and launch shape, in the order of the program (bench.py times a
       configuration as one such run: 20 + 5 x 200 launches over distinct copies, then as many on one copy): calls and
       average duration per run, with the two counters per run when their directories are given
-  python -m trueno_amd.rocprof_summary pmc <dir> [--prefix q4k_gemm] [--min 100]
+  python rocprof_summary.py pmc <dir> [--prefix q4k_gemm] [--min 100]
       every counter of one `--pmc` run, averaged per dispatch over the same runs of consecutive dispatches
+  python rocprof_summary.py timed <dir> --steps K [--ms-per-step T]
+      the dispatches inside the regions bench.py brackets with a 4 KB kq_read_u128 (one workgroup): per region and kernel
+      the calls, the average duration and the kernel time per pass (K passes to a region); with --ms-per-step the check that
+      the kernel time per pass of the first region - the headline's - does not exceed what bench.py reported
 
 The runs (on the GPU box, `cd /tmp && export TMPDIR=/tmp` first):
-  rocprofv3 --kernel-trace --stats -d <dir> -- python3 bench.py --steps 10 --warmup 2 --no-cpu-baseline --no-executors --no-configs
+  rocprofv3 --kernel-trace --stats -d <dir> -- python3 bench.py --steps 20 --warmup 5 --pass-only
   rocprofv3 --pmc FETCH_SIZE -d <fetch_dir> -- python3 bench.py --steps 2 --warmup 1 --pass-only
   rocprofv3 --pmc WRITE_SIZE -d <write_dir> -- python3 bench.py --steps 2 --warmup 1 --pass-only
 """
@@ -170,6 +174,33 @@ def pmc(path: str, prefix: str, least: int) -> None:
         print(f"| {i} | {key[0]} | {key[1]} | {key[2]} | {len(d)} | {vals} |")
 
 
+def timed(path: str, steps: int, ms_per_step: float | None) -> None:
+    for db in _dbs(path):
+        con = sqlite3.connect(db)
+        rows = list(con.execute("select name, grid_x, workgroup_x, start, end from kernels order by start"))
+        marks = [i for i, r in enumerate(rows) if r[0].split("(")[0] == "kq_read_u128" and r[1] == 256]
+        if len(marks) < 2:
+            raise SystemExit("no pair of region marks (kq_read_u128 over 4 KB) in the trace")
+        for region in range(len(marks) // 2):
+            inside = rows[marks[2 * region] + 1:marks[2 * region + 1]]
+            by = {}
+            for name, grid, wg, start, end in inside:
+                by.setdefault((name.split("(")[0], grid, wg), []).append((end - start) / 1e3)
+            # the warm-up passes of a region come before its first mark only in the headline region; a region's first
+            # `len - steps * calls_per_pass` dispatches would be warm-up otherwise: bench.py marks after the warm-up
+            span = (inside[-1][4] - inside[0][3]) / 1e3 if inside else 0.0
+            total = sum(sum(v) for v in by.values())
+            print(f"region {region}: {len(inside)} dispatches, first start to last end {span / steps:.1f} us per pass, "
+                  f"kernel time {total / steps:.1f} us per pass")
+            print("| kernel | grid threads | block | calls | calls per pass | average us | min us | max us | us per pass |")
+            print("|---|---|---|---|---|---|---|---|---|")
+            for key, v in sorted(by.items(), key=lambda kv: -sum(kv[1])):
+                print(f"| {key[0]} | {key[1]} | {key[2]} | {len(v)} | {len(v) / steps:g} | {sum(v) / len(v):.2f} | {min(v):.2f} | {max(v):.2f} | {sum(v) / steps:.1f} |")
+            if region == 0 and ms_per_step is not None:
+                ok = total / steps <= ms_per_step * 1e3
+                print(f"check: kernel time per pass {total / steps:.1f} us {'<=' if ok else '>'} ms_per_step {ms_per_step * 1e3:.1f} us: {'holds' if ok else 'FAILS'}")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -178,7 +209,7 @@ def main() -> int:
     tf = sub.add_parser("traffic")
     tf.add_argument("fetch_dir")
     tf.add_argument("write_dir")
-    tf.add_argument("--kernel", default="kq_gemv_group")
+    tf.add_argument("--kernel", default="kq_gemv_many")
     tf.add_argument("--json")
     sh = sub.add_parser("shapes")
     sh.add_argument("fetch_dir")
@@ -194,8 +225,14 @@ def main() -> int:
     pm.add_argument("dir")
     pm.add_argument("--prefix", default="")
     pm.add_argument("--min", type=int, default=100)
+    tm = sub.add_parser("timed")
+    tm.add_argument("dir")
+    tm.add_argument("--steps", type=int, required=True)
+    tm.add_argument("--ms-per-step", type=float)
     a = ap.parse_args()
-    if a.cmd == "trace":
+    if a.cmd == "timed":
+        timed(a.dir, a.steps, a.ms_per_step)
+    elif a.cmd == "trace":
         trace(a.dir)
     elif a.cmd == "pmc":
         pmc(a.dir, a.prefix, a.min)

@@ -135,7 +135,9 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
 //   LDS: [k floats of x, swizzled][rows_per_block partial sums][64 group sums of squares][ring: waves * 2 * slot bytes]
 // ------------------------------------------------------------------------------------------------------------
 template <int FMT, int U> struct StreamSlot {
-  static constexpr u32 PIECES = (U * 16u * Quarter<FMT>::SB + 15u + 1023u) / 1024u;   // wave instructions per batch
+  // wave instructions per batch: the batch's bytes from the 16-byte boundary below its first one (Q6_K rows can start
+  // at any even address) in KB
+  static constexpr u32 PIECES = (U * 16u * Quarter<FMT>::SB + (FMT == FMT_Q6K ? 15u : 0u) + 1023u) / 1024u;
   static constexpr u32 BYTES = PIECES * 1024u;
 };
 
@@ -176,22 +178,48 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
   // first piece of the matrix (one line, from the cache).  One form for every case, so that a batch is the same
   // number of copies on every path: a branch between forms is two branches in the assembly, with a path that takes
   // neither as far as a reader of the assembly can tell.
+  // Q4_K / Q5_K: rows are whole 16-byte pieces, so a batch starts on a piece and which piece a lane copies with which
+  // instruction is the same for every batch: the offsets are formed once (pieces behind the batch's last repeat it).  A
+  // batch that would reach behind the matrix starts as many rows early instead and its rows are found further into the
+  // slot; one that does not exist reads the matrix's first batch.
+  constexpr bool kPieceAligned = FMT != FMT_Q6K;
+  [[maybe_unused]] u32 piece_off[NL];
+  if constexpr (kPieceAligned) {
+    const u32 last = (batch_bytes - 1u) >> 4;
+#pragma unroll
+    for (u32 j = 0; j < NL; ++j) {
+      const u32 p = 64u * j + lane;
+      piece_off[j] = 16u * (p < last ? p : last);
+    }
+  }
   auto issue = [&](u32 b, u32 slot) -> u32 {
     size_t off = static_cast<size_t>(row0 + b * U) * row_bytes;
     const bool exists = b < batches && off < total;
     if (!exists) off = 0;
-    const u32 avail = static_cast<u32>(total - off < batch_bytes ? total - off : batch_bytes);
-    const uint8_t* src = e.w + off;
-    const u32 shift = static_cast<u32>(reinterpret_cast<size_t>(src)) & 15u;
-    src -= shift;
-    const u32 last = exists ? (shift + avail - 1u) >> 4 : 0u;       // the last 16-byte piece that holds bytes of the batch
     const u32 dst = lds_ring + slot * Slot::BYTES;
+    if constexpr (kPieceAligned) {
+      u32 shift = 0;
+      if (total - off < batch_bytes) {                                // (total >= batch_bytes: the launcher streams no matrix of fewer than U rows)
+        shift = batch_bytes - static_cast<u32>(total - off);
+        off = total - batch_bytes;
+      }
+      const uint8_t* src = e.w + off;
 #pragma unroll
-    for (u32 j = 0; j < NL; ++j) {
-      const u32 p = 64u * j + lane;
-      dma16_nt(src + 16u * (p < last ? p : last), dst + 1024u * j);
+      for (u32 j = 0; j < NL; ++j) dma16_nt(src + piece_off[j], dst + 1024u * j);
+      return shift;
+    } else {
+      const u32 avail = static_cast<u32>(total - off < batch_bytes ? total - off : batch_bytes);
+      const uint8_t* src = e.w + off;
+      const u32 shift = static_cast<u32>(reinterpret_cast<size_t>(src)) & 15u;
+      src -= shift;
+      const u32 last = exists ? (shift + avail - 1u) >> 4 : 0u;       // the last 16-byte piece that holds bytes of the batch
+#pragma unroll
+      for (u32 j = 0; j < NL; ++j) {
+        const u32 p = 64u * j + lane;
+        dma16_nt(src + 16u * (p < last ? p : last), dst + 1024u * j);
+      }
+      return shift;
     }
-    return shift;
   };
 
   // Activations first (loads return in order, and the vector is an L2 hit), then the first two batches of this wave.
@@ -295,8 +323,9 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       const u32 slot = it & 1u;
       const u32 base = lds_ring + slot * Slot::BYTES + shift_cur + sbc * Q::SB;
+      const u32 rows_here = n_dim - (row0 + cur * U);               // (>= 1) rows behind the matrix's last re-read it: never stored
 #pragma unroll
-      for (int u = 0; u < U; ++u) Q::load_lds(regs[u], base + u * row_bytes, c);
+      for (int u = 0; u < U; ++u) Q::load_lds(regs[u], base + (static_cast<u32>(u) < rows_here ? u : rows_here - 1u) * row_bytes, c);
       // the batch after the next: handed out among the waves as they become free (the memory system does not serve
       // them evenly); its copies go where the current batch was, which is in registers when the reads have returned
       u32 nn;
@@ -311,8 +340,8 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       if (more) shift_nn = issue(nn, slot);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
-        if (lane == 0) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_part + 4u * (cur * U + u)), "v"(p) : "memory");
+        const float p = wave_sum_lane63(Q::dot(regs[u], c, xr, sx));
+        if (lane == 63u) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_part + 4u * (cur * U + u)), "v"(p) : "memory");
       }
       cur = nxt; shift_cur = shift_nxt;
       nxt = nn; shift_nxt = shift_nn;
@@ -491,8 +520,8 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
         if (handed_out && lane == 0) nb = __hip_atomic_fetch_add(&s_next[sw], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const float p = wave_sum(Q::dot(regs[u], c, xr, sx));
-          if (lane == 0) {
+          const float p = wave_sum_lane63(Q::dot(regs[u], c, xr, sx));
+          if (lane == 63u) {
             const u32 idx = sw * rows_per_block + b * U + u;
             part[idx] = (slab == sw) ? p : part[idx] + p;
           }

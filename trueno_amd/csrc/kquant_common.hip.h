@@ -79,6 +79,20 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// The same sum, in the same order - ((r3 + r2) + (r1 + r0)) of the four row sums, i.e. wave_sum's bits - but valid in
+// lane 63 only: the rows meet through two broadcasts of a row's last lane into the rows behind it instead of four
+// reads of a lane into scalar registers and three more additions.
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+  v += dpp_f32<0xB1>(v);
+  v += dpp_f32<0x4E>(v);
+  v += dpp_f32<0x141>(v);
+  v += dpp_f32<0x140>(v);
+  // row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3 (lanes not written keep their value)
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));
+  return v;
+}
+
 // ---- byte-wise decoders: one value of one super-block -----------------------------------
 // Used by the generic (any alignment, any K) kernels and by the GEMM-family decode policy.
 // __fmul_rn/__fsub_rn keep every PTX instruction of the reference a separate rounding.

@@ -68,7 +68,7 @@ constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <
 // KQ_U rows of 16 blocks, from the 16-byte boundary below its first byte, in whole KB: StreamSlot of the kernels).
 constexpr uint32_t kChainStreamFlag = 16u;     // CHAIN_STREAM_LDS
 constexpr uint32_t kStreamLdsLimit = 160 * 1024 - 1024;   // dynamic LDS such a launch may ask for (the CU has 160 KB; static LDS is a few words)
-constexpr uint32_t stream_slot_bytes(uint32_t sb_bytes) { return (kGemvRowsPerBatch * 16u * sb_bytes + 15u + 1023u) / 1024u * 1024u; }
+constexpr uint32_t stream_slot_bytes(uint32_t sb_bytes) { return (kGemvRowsPerBatch * 16u * sb_bytes + (sb_bytes == 210u ? 15u : 0u) + 1023u) / 1024u * 1024u; }
 
 struct DeviceKernels {
   bool loaded = false;
@@ -218,8 +218,8 @@ struct GemvGeometry {
 // Q6_K stays on the register path: its 210-byte blocks lie at 2-byte alignment in LDS too, and the five reads per row
 // that start there cost more than the whole-line copies gain (eight 4096 x 4096 per call 3.18 -> 3.38 us a matrix,
 // 32000 x 4096 19.4 -> 19.9 us; Q4_K 11008 x 4096 5.02 -> 4.53 us, Q5_K 6.57 -> 6.29 us).  "gemv_stream_q6k" turns it on.
-bool stream_ok(uint32_t fmt_code, uint32_t k) {
-  return !g_tune_stream_off && k != 0 && k <= 4096u && (fmt_code != 6u || g_tune_stream_q6k);
+bool stream_ok(uint32_t fmt_code, uint32_t k, uint32_t n) {
+  return !g_tune_stream_off && k != 0 && k <= 4096u && n >= kGemvRowsPerBatch && (fmt_code != 6u || g_tune_stream_q6k);
 }
 
 // Geometry of a single streamed GEMV: workgroups of `waves` waves, as many per CU as their LDS allows (two by default).
@@ -573,7 +573,7 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void* gemm_args[] = {&a, &w, &c, &m, &n, &k};
   void** args = is_gemv ? gemv_args : gemm_args;
   GemvGeometry g;
-  if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(uint32_t(f) + 4u, k)) {
+  if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(uint32_t(f) + 4u, k, n)) {
     g = stream_geometry(*d, f, k, n);
     if (g.fits) {
       flags |= kChainStreamFlag;
@@ -1391,7 +1391,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
     const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
     // a streamed entry's bytes arrive faster than those of an entry on the register path
-    const bool streamed = stream_ok(e.fmt, e.k) &&
+    const bool streamed = stream_ok(e.fmt, e.k, e.n) &&
                           uint64_t(e.k) * 4u + kLdsScratch + waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) + kGemvRowsPerBatch * 4u <= kStreamLdsLimit;
     const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
     return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u)) * (streamed ? stream_cost : 1.0);
@@ -1407,7 +1407,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   // an entry of one slab streams its rows through LDS when the rings of all waves fit beside its vector
   auto ring_of = [&](uint32_t i) -> uint32_t {
     const trn_gemv_desc& e = descs[i];
-    if (!stream_ok(e.fmt, e.k)) return 0u;
+    if (!stream_ok(e.fmt, e.k, e.n)) return 0u;
     const uint32_t ring = waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]);
     return uint64_t(e.k) * 4u + kLdsScratch + ring + kGemvRowsPerBatch * 4u <= kStreamLdsLimit ? ring : 0u;
   };
@@ -1520,7 +1520,7 @@ hipError_t plan_gemv_many(DeviceKernels* d, const trn_gemv_desc* descs, uint32_t
   for (uint32_t i = 0; i < len; ++i) {
     const trn_gemv_desc& e = descs[i];
     const uint32_t slabs = (e.k / 256u + 15u) / 16u, sw = std::min(slabs, waves);
-    uint32_t ring = stream_ok(e.fmt, e.k) ? waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) : 0u;
+    uint32_t ring = stream_ok(e.fmt, e.k, e.n) ? waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) : 0u;
     const uint64_t x_bytes = uint64_t(e.k) * 4u;
     if (ring && x_bytes + kLdsScratch + ring + ug * 4u > kStreamLdsLimit) ring = 0u;
     const uint64_t limit = ring ? kStreamLdsLimit - ring : kFastLdsLimit;
@@ -1596,9 +1596,14 @@ struct PlannedLaunch {
 struct ListPlan {
   std::vector<trn_gemv_desc> key;
   int epoch = -1;
+  uint64_t used = 0;           // when it was used last (g_plan_clock)
   std::vector<PlannedLaunch> launches;
 };
-std::map<std::tuple<int, hipStream_t, bool>, ListPlan> g_list_plans;     // by device, stream and "may make large launches"; under g_ws_mutex
+// A few plans per stream (a decoder may issue the layers' lists one by one, or alternate between lists): the one used
+// longest ago makes room for a new list.
+constexpr size_t kPlansPerStream = 8;
+uint64_t g_plan_clock = 0;
+std::map<std::tuple<int, hipStream_t, bool>, std::vector<ListPlan>> g_list_plans;     // by device, stream and "may make large launches"; under g_ws_mutex
 
 void free_plan_tables(ListPlan* plan) {
   for (PlannedLaunch& l : plan->launches)
@@ -1610,7 +1615,7 @@ void free_plan_tables(ListPlan* plan) {
 void release_list_plans(hipStream_t stream) {       // under g_ws_mutex; the stream is idle
   for (auto it = g_list_plans.begin(); it != g_list_plans.end();) {
     if (std::get<1>(it->first) == stream) {
-      free_plan_tables(&it->second);
+      for (ListPlan& p : it->second) free_plan_tables(&p);
       it = g_list_plans.erase(it);
     } else {
       ++it;
@@ -1712,9 +1717,23 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
   }
   const bool many_ok = capturing == hipStreamCaptureStatusNone;
   std::lock_guard<std::mutex> lock(g_ws_mutex);
-  ListPlan& plan = g_list_plans[std::make_tuple(dev, stream, many_ok)];      // (a capture has a plan of its own)
-  const bool same = plan.epoch == g_tune_epoch && plan.key.size() == count &&
-                    std::memcmp(plan.key.data(), descs, size_t(count) * sizeof(trn_gemv_desc)) == 0;
+  std::vector<ListPlan>& plans = g_list_plans[std::make_tuple(dev, stream, many_ok)];      // (a capture has plans of its own)
+  ListPlan* found = nullptr;
+  for (ListPlan& p : plans)
+    if (p.epoch == g_tune_epoch && p.key.size() == count && std::memcmp(p.key.data(), descs, size_t(count) * sizeof(trn_gemv_desc)) == 0) found = &p;
+  const bool same = found != nullptr;
+  if (!same) {
+    if (plans.size() < kPlansPerStream) {
+      plans.emplace_back();
+      found = &plans.back();
+    } else {
+      found = &plans[0];
+      for (ListPlan& p : plans)
+        if (p.used < found->used) found = &p;
+    }
+  }
+  ListPlan& plan = *found;
+  plan.used = ++g_plan_clock;
   if (!same) {
     bool had_tables = false;
     for (const PlannedLaunch& l : plan.launches) had_tables = had_tables || l.many.dev;
