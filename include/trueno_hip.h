@@ -14,9 +14,16 @@
  * reference maps any non-zero CUresult to GpuError::CudaDriver(name, code), sys.rs:360-369; a missing
  * device is hipErrorNoDevice = 100, which maps to GpuError::CudaNotAvailable).  Device pointers
  * are plain 64-bit integers (CUdeviceptr, sys.rs:60).  The library never owns host memory and never
- * keeps a host pointer after a synchronous call returns.  Nothing here allocates device memory
- * except trn_mem_alloc.  All entry points may be called from any thread; calls that touch a device
- * act on the calling thread's current device (trn_ctx_set_current).
+ * keeps a host pointer after a synchronous call returns.  Device memory for the caller's data comes
+ * from trn_mem_alloc only.  Beside it the library keeps scratch of its own, per (device, stream),
+ * allocated on first use and freed with the stream: the partial sums and arrival counters of the
+ * products that are cut along K (trn_q*k_gemm, trn_gemv_f32, trn_incremental_attention), the tables
+ * of a list's launches of more than sixteen entries (trn_kquant_gemv_batch), the tables of the
+ * resident executor (batch_mode 1); and one static array of 16 MiB + 64 KiB per GPU
+ * (trn_q4k_gemm_noalloc).  The calls that never allocate: the GEMV launchers, trn_kquant_gemv_batch
+ * for lists whose launches hold at most sixteen entries or while the stream is being captured,
+ * trn_q4k_gemm_noalloc, the element-wise launchers.  All entry points may be called from any thread;
+ * calls that touch a device act on the calling thread's current device (trn_ctx_set_current).
  */
 #ifndef TRUENO_HIP_H
 #define TRUENO_HIP_H
@@ -81,7 +88,10 @@ TRN_API trn_status trn_module_get_function(trn_function* func, trn_module module
  * set on the function handle (one module per kernel instance, as in the reference) before it is launched by name with
  * the reference's own parameter list: "rmsnorm" (input, output, gamma), "fused_residual_rmsnorm" (residual, input,
  * output, gamma), "incremental_attention" (q, k, v, out, seq_len).  Launching one of these by name without its
- * constants returns TRN_ERROR_INVALID_VALUE; nothing beyond the reference's parameters is ever read. */
+ * constants returns TRN_ERROR_INVALID_VALUE; nothing beyond the reference's parameters is ever read.  The constants
+ * belong to the one handle that trn_module_get_function returns for (module, name): two kernel instances with
+ * different constants need a module each, and a thread that sets a handle while another launches it must be kept
+ * apart from it by the caller (a set is two or five plain stores). */
 TRN_API trn_status trn_function_set_rmsnorm(trn_function func, uint32_t hidden_size, float epsilon);
 TRN_API trn_status trn_function_set_attention(trn_function func, uint32_t head_dim, uint32_t num_heads,
                                               uint32_t num_kv_heads, uint32_t max_seq_len, float scale);
@@ -148,10 +158,11 @@ TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant,
  * results of the parts of K and their arrival counters), this entry point uses a buffer that is part of the library
  * image: a static device array of 16 MiB + 64 KiB, of which every GPU the library runs on holds one copy until the
  * process ends.  After the library's first use on the device (any launcher, or trn_ctx_set_current, loads the kernels
- * and looks the buffer's address up once) it calls nothing that allocates or frees.  A product that needs more
- * scratch than that returns TRN_ERROR_SCRATCH_TOO_SMALL and launches nothing (every cut of a product that the library
- * chooses by itself needs at most 11.2 MB on 256 CUs; a cut forced with trn_set_tuning may need more, and the library then
- * takes one that fits if there is one; m = 1 and unaligned operands take kernels that need no scratch).  All calls on
+ * and looks the buffer's address up once) it calls nothing that allocates or frees.  The product is cut exactly as
+ * trn_q4k_gemm would cut it - hence the same bits - and when that cut needs more scratch than the buffer holds the call
+ * returns TRN_ERROR_SCRATCH_TOO_SMALL and launches nothing; no other failure is reported under that name (every cut that
+ * the library chooses by itself needs at most 11.2 MB on 256 CUs; a cut forced with trn_set_tuning may need more; m = 1
+ * and unaligned operands take kernels that need no scratch).  All calls on
  * one GPU share that GPU's buffer: calls that overlap in time on different streams of one GPU race - keep them on
  * one stream, or order the streams.  The kernels leave the counters at zero for the next call. */
 TRN_API trn_status trn_q4k_gemm_noalloc(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
@@ -176,10 +187,15 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * roadmap.yaml:359-368).  Entry i computes y = dequant(W) x exactly as the typed launcher of its
  * format would; a later entry may read what an earlier one wrote (the library finds those
  * dependencies from the pointer ranges).  fmt: 4 = Q4_K, 5 = Q5_K, 6 = Q6_K.
- * By default (mode 0) entries that do not touch one another's vectors share a launch, up to eight: the first
- * entry still waiting, plus later ones of a window of the list (q, k, v of a decoder layer; gate and up; ...)
- * that depend neither on it nor on anything they would overtake.  What an entry computes does not depend on the
- * company it is launched in: the results are, bit for bit, those of one launch per entry in list order.
+ * By default (mode 0) entries that do not touch one another's vectors share a launch: the first entry still
+ * waiting, plus every later one of the list (q, k, v of a decoder layer; gate and up; the same of other layers
+ * when each layer has activation buffers of its own; ...) that depends neither on it nor on anything it would
+ * overtake.  Up to sixteen entries travel in the kernel's arguments; a launch of more takes them from tables in
+ * device memory, which are made when a list is first seen on a stream and kept for as long as the same list (the
+ * same descriptors, byte for byte) comes again - up to eight lists per stream, the one used longest ago makes room.
+ * While the stream is being captured into a graph launches hold at most sixteen entries (nothing is copied or
+ * allocated).  What an entry computes does not depend on the company it is launched in: the results are, bit for
+ * bit, those of one launch per entry in list order.
  * With trn_set_tuning("batch_mode", 1), and when every entry meets the fast kernels' alignment (x 16 B,
  * W 16 B / 2 B for Q6_K), the list runs as ONE cooperative launch of resident workgroups: the list is cut in
  * phases of mutually independent entries with a device-side barrier between phases.  This form keeps, per
@@ -277,7 +293,7 @@ TRN_API trn_status trn_fused_residual_rmsnorm(trn_stream stream, trn_dptr residu
 /* dst[0..bytes) = src[0..bytes) with one 16-byte load and store per lane; bytes % 16 == 0.
  * The plain-copy yardstick that HBM counters are scaled by. */
 TRN_API trn_status trn_copy_u128(trn_stream stream, trn_dptr dst, trn_dptr src, uint64_t bytes);
-/* Reads src[0..bytes) once with 16-byte loads, eight in flight per lane, and stores nothing (one word of `sink`, 4 bytes,
+/* Reads src[0..bytes) once with non-temporal 16-byte loads, eight in flight per lane, and stores nothing (one word of `sink`, 4 bytes,
  * is written only if the XOR of everything read equals one particular value); bytes % 16 == 0.  The read-only
  * yardstick: what one launch over that many bytes costs when nothing is computed.  No counterpart in the reference. */
 TRN_API trn_status trn_read_u128(trn_stream stream, trn_dptr src, uint64_t bytes, trn_dptr sink);
@@ -289,10 +305,17 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * geometry of the single-GEMV kernels.  "batch_mode": how trn_kquant_gemv_batch runs a list - 0 grouped
  * launches (default), 1 one cooperative launch of resident workgroups with device-side barriers.
  * "chain_spin_limit": polls a device-side barrier wait may take before it gives up.
- * "group_off": 1 = in mode 0 one launch per entry; "group_max": most entries in a launch (0 = 16, the most the kernel holds); "group_window":
- * how far down the list a launch looks for entries (0 = 32); "group_waves": least waves per workgroup of such a launch (0 = what
- * its widest entry needs); "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch
- * shares out its workgroups (0 = 40).
+ * "group_off": 1 = in mode 0 one launch per entry; "group_max": most entries in a launch (0 = as many as the list offers,
+ * up to 4096; 16 or less keeps every launch on the kernel-argument form); "group_window": how far down the list a launch
+ * looks for entries (0 = twice group_max); "group_waves": least waves per workgroup of a launch of up to sixteen entries (0 = 8,
+ * or what its widest entry needs); "many_waves": waves per workgroup of a launch of more than sixteen entries (0 = 12);
+ * "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch shares out its
+ * workgroups (0 = 40).
+ * "gemv_stream_off": 1 = no matrix streams its rows through LDS (every GEMV loads its rows into registers straight from
+ * memory; same bits); "gemv_stream_q6k": 1 = Q6_K matrices of up to 4096 columns stream too (slower, measured);
+ * "gemv_stream_waves": waves per workgroup of a single streamed GEMV (0 = 4); "gemv_stream_min_rows": a single GEMV
+ * streams when a wave gets at least this many rows (0 = 16); "gemv_stream_cost": percent of its bytes a streamed entry
+ * counts for when a launch shares out its workgroups (0 = 95).
  * "gemm_mfma_off": 1 = the k-quant GEMMs never take the matrix-core form; "gemm_k_parts": into how many parts
  * that form cuts K; "gemm_waves": 4, 8 or (Q4_K) 12 strips of 32 rows per workgroup; "gemm_tiles": 1 or 2 tiles of 16 tokens per
  * workgroup (0 for each of the three = chosen from the shape by an estimated time; any of them set also keeps a

@@ -79,7 +79,15 @@ def test_host_side_transfer_checks_need_no_driver():
     empty.copy_from_host(np.zeros(0, np.float32))
     assert empty.copy_to_host().size == 0
     meta = buf.clone_metadata()
-    assert meta.as_ptr() == 0x1000 and meta.len() == 8 and meta.size_bytes() == 32
+    assert isinstance(meta, t.GpuBufferView) and meta.as_ptr() == 0x1000 and meta.len() == 8 and meta.size_bytes() == 32 and not meta.is_empty()
+    other = t.GpuBuffer.from_raw_parts(0x2000, 4, np.float32)
+    with pytest.raises(t.GpuError) as e:                       # memory.rs:583-594: bounds are checked before any driver call
+        buf.copy_from_buffer_at_async_raw(other, 6, 0, 3, None)
+    assert e.value.kind == "Transfer" and "dst out of bounds: 6 + 3 > 8" in str(e.value)
+    with pytest.raises(t.GpuError) as e:
+        buf.copy_from_buffer_at_async_raw(other, 0, 2, 3, None)
+    assert e.value.kind == "Transfer" and "src out of bounds: 2 + 3 > 4" in str(e.value)
+    buf.copy_from_buffer_at_async_raw(other, 0, 0, 0, None)    # nothing to copy: no driver call
     assert buf.as_kernel_arg().value == 0x1000
     with pytest.raises(t.GpuError) as e:
         t.QuantizeKernel(1, 1, 32).launch(None, 0, 0, 0)

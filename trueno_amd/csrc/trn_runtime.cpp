@@ -105,10 +105,10 @@ std::atomic<int> g_tune_gemm_mfma_off{0};   // 1: the Q4_K GEMM never takes the 
 std::atomic<int> g_tune_gemm_tiles{0};      // token tiles per workgroup of the matrix-core GEMM: 0 by the rule, 1, 2
 std::atomic<int> g_tune_gemm_ksplit{0};     // parts of K in the matrix-core GEMM (0: chosen from the shape)
 std::atomic<int> g_tune_attention_min_steps{0};
-std::atomic<int> g_tune_group_window{0};       // entries of a list a grouped launch may look ahead over (0: 16)
-std::atomic<int> g_tune_group_waves{0};        // least waves per workgroup of a grouped launch (0: what the widest entry needs)
-std::atomic<int> g_tune_group_max{0};          // most entries in one grouped launch (0: 8; at most 16)
-std::atomic<int> g_tune_slab_weight{0};        // percent a grouped launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 30)
+std::atomic<int> g_tune_group_window{0};       // entries of a list a launch may look ahead over (0: twice the most it may hold)
+std::atomic<int> g_tune_group_waves{0};        // least waves per workgroup of a launch of up to sixteen entries (0: 8, or what the widest entry needs)
+std::atomic<int> g_tune_group_max{0};          // most entries in one launch (0: as many as the list offers, up to kManyMax)
+std::atomic<int> g_tune_slab_weight{0};        // percent a launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: 40)
 std::atomic<int> g_tune_attention_per_cu{0};   // workgroups per CU the single-query attention aims at (0: default)
 std::atomic<int> g_tune_gemm_waves{0};      // strips of 32 rows per workgroup of the matrix-core GEMM: 4, 8 or (Q4_K) 12 (0: default)
 std::atomic<int> g_tune_stream_off{0};      // 1: one-slab GEMVs load their rows into registers straight from memory (no LDS ring)
@@ -501,14 +501,14 @@ GemmCut gemm_cut(const DeviceKernels& d, Fmt f, uint32_t m, uint32_t n, uint32_t
 // ext_base != 0: the caller brings the scratch buffer (ext_cap bytes, counters at its front already zero); nothing is
 // allocated and a product that needs more is refused.
 hipError_t launch_kq_gemm_f16(DeviceKernels* d, Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m,
-                              uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0) {
+                              uint32_t n, uint32_t k, uint64_t ext_base = 0, size_t ext_cap = 0, const GemmCut* given = nullptr) {
   const uint32_t nsb = k / 256u, tiles = (m + 15u) / 16u;
   const uint32_t kGemmWTileBytes = 32u * kSbBytes[f];
   // Q6_K: one weight tile per wave, rows 240 bytes apart (q6k_lds_bytes of the kernel's header)
   const uint32_t kGemmQ6TileBytes = 32u * 240u;
   // a caller's own scratch buffer: only cuts whose partial sums fit behind the counters
   const size_t part_cap = ext_base == 0 ? ~size_t(0) : ext_cap > kGemmCounterBytes ? ext_cap - kGemmCounterBytes : 0u;
-  const GemmCut cut = gemm_cut(*d, f, m, n, k, part_cap);
+  const GemmCut cut = given ? *given : gemm_cut(*d, f, m, n, k, part_cap);
   const uint32_t waves = cut.waves, nt = cut.nt, groups = cut.groups, tgroups = cut.tgroups, kparts = cut.kparts, ksb = cut.ksb;
   const uint32_t lds = f == Q6K ? 2u * kGemmXpStageBytes + waves * kGemmQ6TileBytes + 16u
                                 : 2u * nt * kGemmXpStageBytes + 2u * waves * kGemmWTileBytes + 16u;
@@ -1809,10 +1809,11 @@ trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c
   size_t cap = 0;
   const uint64_t base = trn_noalloc_scratch(dev, &cap);
   if (!base) return TRN_ERROR_INVALID_VALUE;
-  // launch_q4k_gemm_f16 answers hipErrorInvalidValue when the product needs more than `cap`: name that case
-  const hipError_t e = launch_kq_gemm_f16(d, Q4K, stream, a, b, c, m, n, k, base, cap);
-  if (e == hipErrorInvalidValue) return TRN_ERROR_SCRATCH_TOO_SMALL;
-  return st(e);
+  // the cut trn_q4k_gemm would take (so the bits are its bits): refused by name when its partial sums do not fit
+  const GemmCut cut = gemm_cut(*d, Q4K, m, n, k);
+  const size_t part_bytes = gemm_part_bytes(cut.kparts, (m + 15u) / 16u, cut.groups, cut.waves);
+  if (kGemmCounterBytes + part_bytes > cap) return TRN_ERROR_SCRATCH_TOO_SMALL;
+  return st(launch_kq_gemm_f16(d, Q4K, stream, a, b, c, m, n, k, base, cap, &cut));
 }
 
 // ---- 9. dequantise test surface ----------------------------------------------------------

@@ -267,8 +267,9 @@ class GpuBuffer:
     def from_raw_parts(ptr: int, length: int, dtype=np.float32) -> "GpuBuffer":
         return GpuBuffer(None, length, dtype, _ptr=ptr)
 
-    def clone_metadata(self) -> "GpuBuffer":
-        return GpuBuffer.from_raw_parts(self._ptr, self._len, self.dtype)
+    def clone_metadata(self) -> "GpuBufferView":
+        """A view of the same device memory that owns nothing (memory.rs:148-170)."""
+        return GpuBufferView(self._ptr, self._len, self.dtype)
 
     def as_ptr(self) -> int:
         return self._ptr
@@ -356,6 +357,20 @@ class GpuBuffer:
             it = self.dtype.itemsize
             _check(_lib().trn_memcpy_dtod(self._ptr + dst_offset * it, src._ptr + src_offset * it, count * it), "Transfer")
 
+    def copy_from_buffer_at_async(self, src: "GpuBuffer", dst_offset: int, src_offset: int, count: int, stream: CudaStream) -> None:
+        """memory.rs:574-611: both buffers must stay valid until the stream has been synchronised."""
+        self.copy_from_buffer_at_async_raw(src, dst_offset, src_offset, count, stream.raw())
+
+    def copy_from_buffer_at_async_raw(self, src: "GpuBuffer", dst_offset: int, src_offset: int, count: int, stream_handle) -> None:
+        """memory.rs:613-650: the same with the raw stream handle."""
+        if dst_offset + count > self._len:
+            raise GpuError("Transfer", f"Async D2D dst out of bounds: {dst_offset} + {count} > {self._len}")
+        if src_offset + count > src._len:
+            raise GpuError("Transfer", f"Async D2D src out of bounds: {src_offset} + {count} > {src._len}")
+        if count:
+            it = self.dtype.itemsize
+            _check(_lib().trn_memcpy_dtod_async(self._ptr + dst_offset * it, src._ptr + src_offset * it, count * it, stream_handle), "Transfer")
+
     def free(self) -> None:
         if self._owned and self._ptr:
             _lib().trn_mem_free(self._ptr)
@@ -367,3 +382,25 @@ class GpuBuffer:
             self.free()
         except Exception:
             pass
+
+
+class GpuBufferView:
+    """Non-owning view of a device buffer (memory.rs:172-207): a pointer and a length, nothing is freed with it."""
+
+    def __init__(self, ptr: int, length: int, dtype=np.float32):
+        self._ptr, self._len, self.dtype = int(ptr), int(length), np.dtype(dtype)
+
+    def as_ptr(self) -> int:
+        return self._ptr
+
+    def len(self) -> int:
+        return self._len
+
+    def __len__(self) -> int:
+        return self._len
+
+    def is_empty(self) -> bool:
+        return self._len == 0
+
+    def size_bytes(self) -> int:
+        return self._len * self.dtype.itemsize
