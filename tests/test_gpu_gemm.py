@@ -291,3 +291,90 @@ def test_gemm_on_streams_that_come_and_go(gpu):
         first = c if first is None else first
         assert np.array_equal(c.view(np.uint32), first.view(np.uint32))
         stream.destroy()
+
+
+# ---- two to four tokens on the integer matrix cores (Q4_K, k <= 4096) --------------------------------------------------
+FEW_SHAPES = [(64, 256), (100, 1024), (33, 2304), (1000, 4096), (8300, 4096), (14336, 4096)]
+
+
+@pytest.mark.parametrize("m", (2, 3, 4))
+@pytest.mark.parametrize("n,k", FEW_SHAPES)
+def test_gemm_few_tokens_on_the_integer_cores(gpu, n, k, m):
+    """One to 260 tiles of 32 rows (one or two per workgroup, the last one ragged), one to sixteen super-blocks per row,
+    every token count the kernel takes: within the contract's distance of fp64, and not the result of another path."""
+    buf, a = kq.gen_matrix("q4k", 600 + m, n, k), kq.gen_x(700 + m, m, k)
+    want = _c64("q4k", buf, a, n, k)
+    try:
+        _tune("gemm_few", 1)
+        c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+        _tune("gemm_few", 2)
+        other = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    finally:
+        _tune("gemm_few", 0)
+    assert c.shape == (m, n) and np.all(np.isfinite(c))
+    assert kq.rel_l2(c, want) <= TOL and kq.rel_l2(other, want) <= TOL
+    assert not np.array_equal(c, other)                      # (two orders of summation: the same bits would mean one path ran twice)
+
+
+@pytest.mark.parametrize("m", (2, 4))
+def test_gemm_few_tokens_no_worse_than_reference_order_f32(gpu, coracle, m):
+    n, k = 2048, 4096
+    buf, a = kq.gen_matrix("q4k", 93, n, k), kq.gen_x(94, m, k)
+    c64 = kq.gemm_fp64(a, kq.dequant_matrix("q4k", buf, n, k))
+    try:
+        _tune("gemm_few", 1)
+        c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    finally:
+        _tune("gemm_few", 0)
+    ref = np.stack([coracle.gemv_ref_order_f32("q4k", buf, a[i], k, n) for i in range(m)])
+    err_ref, err_ours = kq.rel_l2(ref, c64), kq.rel_l2(c, c64)
+    record_ratio("gemm_few", "q4k", m, n, k, n, err_ours, err_ref)
+    assert err_ours <= REF_SLACK * err_ref, (m, err_ours, err_ref, err_ours / err_ref)
+
+
+def test_gemm_few_tokens_special_values(gpu):
+    """Tokens of zeros, of huge and of tiny values; a token whose runs of 256 differ by 2^40 in size and one with a single
+    large element among small ones (each run has its own power of two, so the small ones keep their bits); unit vectors
+    (the product is then one weight, d * s * q - dmin * m, to a few ulps of its two terms); an infinity spoils its
+    token and no other."""
+    n, k = 96, 1024
+    buf = kq.gen_matrix("q4k", 95, n, k)
+    w = kq.dequant_matrix("q4k", buf, n, k)
+    a = kq.gen_x(96, 4, k)
+    a[1] = 0.0
+    a[2] *= 1e30
+    a[3, :256] *= 2.0 ** 40
+    a[3, 700] = 3.0e4
+    try:
+        _tune("gemm_few", 1)
+        c = gpu_gemm(gpu, "q4k", buf, a, 4, n, k)
+        a2 = kq.gen_x(97, 3, k) * 1e-30
+        a2[1] = 0.0
+        a2[1, 517] = 1.0
+        a2[2, 3] = np.inf
+        c2 = gpu_gemm(gpu, "q4k", buf, a2.astype(np.float32), 3, n, k)
+    finally:
+        _tune("gemm_few", 0)
+    c64 = kq.gemm_fp64(a, w)
+    assert np.all(c[1] == 0.0)
+    for i in (0, 2, 3):
+        assert kq.rel_l2(c[i], c64[i]) <= TOL
+    assert kq.rel_l2(c2[0], kq.gemm_fp64(a2[:1].astype(np.float32), w)[0]) <= TOL
+    col = w[:, 517].astype(np.float64)
+    assert np.all(np.abs(c2[1] - col) <= 2.0 ** -21 * np.abs(w).max())
+    assert not np.any(np.isfinite(c2[2]))
+
+
+def test_gemm_few_tokens_by_the_rule(gpu):
+    """Left to itself the launcher takes the integer-core kernel where it is the fastest way (two tokens against 14336
+    rows), and not for one token, for five, or for rows longer than a slab of 4096 columns."""
+    for m, n, k, taken in [(2, 14336, 4096, True), (1, 2048, 4096, False), (5, 2048, 4096, False), (2, 256, 8192, False)]:
+        buf, a = kq.gen_matrix("q4k", 31 + m, n, k), kq.gen_x(32 + m, m, k)
+        c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+        try:
+            _tune("gemm_few", 2)
+            other = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+        finally:
+            _tune("gemm_few", 0)
+        assert kq.rel_l2(c, _c64("q4k", buf, a, n, k)) <= TOL
+        assert np.array_equal(c, other) != taken, (m, n, k)

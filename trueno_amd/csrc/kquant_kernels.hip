@@ -13,6 +13,7 @@
 #endif
 #include "kquant_chain.hip.h"
 #include "kquant_gemm_f16.hip.h"
+#include "kquant_few_i8.hip.h"
 #include "decode_glue.hip.h"
 #include "gemv_f32.hip.h"
 #include "decode_attention.hip.h"
@@ -343,6 +344,21 @@ KQ_GEMM_F16(q4k_gemm_f16_w8t2, 512, kq_body<FMT_Q4K KQ_COMMA 8 KQ_COMMA 2>)
 KQ_GEMM_F16(q5k_gemm_f16_w8t2, 512, kq_body<FMT_Q5K KQ_COMMA 8 KQ_COMMA 2>)
 KQ_GEMM_F16(q6k_gemm_f16_w8, 512, q6k_body<1>)
 KQ_GEMM_F16(q6k_gemm_f16_w4, 256, q6k_body<2>)
+
+// Q4_K product for two to four tokens on the integer matrix cores (kquant_few_i8.hip.h): workgroup b takes the rows
+// b * rows_per_wg .. of W, k <= 4096.
+#define KQ_GEMM_FEW(name, NTOK)                                                                                          \
+  extern "C" __global__ void __launch_bounds__(512)                                                                      \
+  name(const float* a, const uint8_t* w, float* c, u32 m, u32 n, u32 k, u32 rows_per_wg) {                               \
+    extern __shared__ uint8_t few_lds[];                                                                                 \
+    const u32 lds_base =                                                                                                 \
+        static_cast<u32>(reinterpret_cast<size_t>((const __attribute__((address_space(3))) uint8_t*)few_lds));          \
+    const u32 row0 = blockIdx.x * rows_per_wg;                                                                           \
+    if (row0 >= n) return;                                                                                               \
+    few_i8::q4k_rows<NTOK>(a, w, c, m, n, k, row0, min(rows_per_wg, n - row0), lds_base);                                \
+  }
+KQ_GEMM_FEW(q4k_gemm_few_t2, 2)
+KQ_GEMM_FEW(q4k_gemm_few_t4, 4)
 
 // Legacy "simplified" Q4_K (trueno-gpu/src/kernels/quantize.rs:151-336, kernel name q4k_gemm_fused): blocks of 32
 // values in 18 bytes - f16 scale at 0, 16 bytes of nibbles at 2, value i in byte i/2 (low nibble for even i);

@@ -86,6 +86,7 @@ struct DeviceKernels {
   hipFunction_t gemm_f16[NFMT][2] = {};   // [format][4 or 8 strips per workgroup]
   hipFunction_t gemm_f16_w12 = nullptr;   // Q4_K: 12 strips per workgroup
   hipFunction_t gemm_f16_t2[2] = {};      // Q4_K, Q5_K: 8 strips and two token tiles per workgroup
+  hipFunction_t gemm_few[2] = {};         // Q4_K, integer matrix cores, built for 2 and 4 tokens
   hipFunction_t gemm_simplified = nullptr, dequant_simplified = nullptr;
 };
 
@@ -117,6 +118,7 @@ std::atomic<int> g_tune_stream_cost{0};     // percent of its bytes a streamed e
 std::atomic<int> g_tune_stream_min_rows{0}; // a single GEMV streams when a wave gets at least this many rows (0: default)
 std::atomic<int> g_tune_many_waves{0};      // waves per workgroup of a launch of more than sixteen entries (0: 12)
 std::atomic<int> g_tune_stream_waves{0};    // waves per workgroup of a single streamed GEMV (0: default)
+std::atomic<int> g_tune_gemm_few{0};        // the integer matrix-core kernel for two to four tokens: 0 by the rule, 1 wherever it can run, 2 never
 
 inline trn_status st(hipError_t e) { return static_cast<trn_status>(e); }
 
@@ -181,6 +183,8 @@ hipError_t device_kernels(DeviceKernels** out) {
         (e = get_fn(m, &t.gemm_f16_t2[1], "q5k_gemm_f16_w8t2")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][0], "q6k_gemm_f16_w4")) != hipSuccess ||
         (e = get_fn(m, &t.gemm_f16[2][1], "q6k_gemm_f16_w8")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_few[0], "q4k_gemm_few_t2")) != hipSuccess ||
+        (e = get_fn(m, &t.gemm_few[1], "q4k_gemm_few_t4")) != hipSuccess ||
         (e = get_fn(m, &t.fill_u32, "kq_fill_u32")) != hipSuccess) {
       (void)hipModuleUnload(m);
       return e;
@@ -556,6 +560,31 @@ bool gemm_few_tokens_by_engine(const DeviceKernels& d, Fmt f, uint32_t m, uint32
   return 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15) < matrix_cores;
 }
 
+// The integer matrix-core kernel (kquant_few_i8.hip.h): Q4_K, two to four tokens, a row of W within one slab of 4096
+// columns.  One workgroup per CU at most (its LDS), each with a run of rows that is a multiple of the tile's 32.
+// Times in microseconds measured on MI355X (cold weights, k = 4096; n = 1024, 4096, 11008, 14336, 32000): two tokens
+// 6.4, 6.7, 10.3, 11.2, 19.0; four tokens 8.4, 8.6, 12.6, 13.1, 21.4 - about 2.1 + 0.7 m (m = 2 or 4: what the kernel is
+// built for) to make the digits and for the launch, and 4 per tile of 32 rows that a workgroup takes.  The other ways took, for two and four tokens, 4.9 / 5.1 (the
+// GEMV engine, a pass per token), 7.2 / 9.2, 12.0 / 14.6, 14.8 / 14.8, 23.4 / 23.6 (the f16 matrix-core form).
+constexpr uint32_t kFewRowPad = 32u;
+double gemm_few_us(const DeviceKernels& d, uint32_t m, uint32_t n) {
+  const uint32_t tiles = (n + 31u) / 32u, wgs = std::min<uint32_t>(tiles, uint32_t(d.cu_count));
+  return 2.1 + 0.7 * (m <= 2u ? 2.0 : 4.0) + 4.0 * ((tiles + wgs - 1u) / wgs);
+}
+bool gemm_few_ok(Fmt f, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  return f == Q4K && g_tune_gemm_few != 2 && m >= 2u && m <= 4u && k != 0 && k <= 4096u && n != 0 && aligned(a, 16) && aligned(w, 16) &&
+         aligned(c, 4);
+}
+hipError_t launch_gemm_few(DeviceKernels* d, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  const uint32_t nsb = k / 256u, idx = m <= 2u ? 0u : 1u, ntok = 2u << idx;
+  const uint32_t tiles = (n + 31u) / 32u, wgs = std::min<uint32_t>(tiles, uint32_t(d->cu_count));
+  uint32_t rows_per_wg = (tiles + wgs - 1u) / wgs * 32u;
+  const uint32_t grid = (n + rows_per_wg - 1u) / rows_per_wg;
+  const uint32_t lds = 2u * 32u * (nsb * 144u + kFewRowPad) + 8u * 32u * ntok * 4u + ntok * nsb * 9u * 4u;
+  void* args[] = {&a, &w, &c, &m, &n, &k, &rows_per_wg};
+  return hipModuleLaunchKernel(d->gemm_few[idx], grid, 1, 1, 512, 1, 1, lds, stream, args, nullptr);
+}
+
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
                             uint32_t k, bool is_gemv, uint32_t flags = 0) {
   if (k % 256u != 0) return hipErrorInvalidValue;
@@ -564,6 +593,13 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
+  if (!is_gemv && gemm_few_ok(f, a, w, c, m, n, k)) {
+    // against the faster of the other two ways, by their fitted times (gemm_few_tokens_by_engine)
+    const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
+    const double engine = 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15);
+    const double cores = !q4k_gemm_f16_ok(a, w, c, m, n, k, f) ? 1e30 : gemm_cut(*d, f, m, n, k).waves == 4u ? 7.2 + mb / 4.0 : 12.0 + mb / 9.4;
+    if (g_tune_gemm_few == 1 || gemm_few_us(*d, m, n) < std::min(engine, cores)) return launch_gemm_few(d, stream, a, w, c, m, n, k);
+  }
   if (!is_gemv && q4k_gemm_f16_ok(a, w, c, m, n, k, f) &&
       (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0 || !gemm_few_tokens_by_engine(*d, f, m, n, k)))
     return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
@@ -1932,6 +1968,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemv_stream_q6k")) { g_tune_stream_q6k = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_cost")) { g_tune_stream_cost = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_min_rows")) { g_tune_stream_min_rows = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "gemm_few")) { g_tune_gemm_few = value; return TRN_SUCCESS; }
   return TRN_ERROR_INVALID_VALUE;
 }
 
