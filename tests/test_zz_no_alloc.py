@@ -41,6 +41,9 @@ def test_noalloc_gemm_equals_the_allocating_entry_point_twice_in_a_row(gpu):
     # m = 1 and unaligned operands take the kernels without scratch: still the same results
     got, want, ref = _both(gpu, 1, 257, 512, 920)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) and kq.rel_l2(got, ref) <= TOL
+    # so do three tokens against 14336 rows (the integer matrix cores: no scratch either)
+    got, want, ref = _both(gpu, 3, 14336, 4096, 940)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)) and kq.rel_l2(got, ref) <= TOL
 
 
 def test_noalloc_gemm_refuses_what_does_not_fit(gpu):

@@ -585,6 +585,23 @@ hipError_t launch_gemm_few(DeviceKernels* d, hipStream_t stream, uint64_t a, uin
   return hipModuleLaunchKernel(d->gemm_few[idx], grid, 1, 1, 512, 1, 1, lds, stream, args, nullptr);
 }
 
+// Which kernel takes a product of m >= 1 tokens: the integer matrix cores (Q4_K, two to four tokens, where their fitted
+// time is below the other ways'), the f16 matrix cores, or the GEMV engine with a pass per token (also: whatever the
+// matrix-core forms cannot take).  A forced cut of the f16 form (tuning) takes that form.
+enum class GemmRoute { kFew, kCores, kOther };
+GemmRoute gemm_route(const DeviceKernels& d, Fmt f, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n, uint32_t k) {
+  const bool cores_ok = q4k_gemm_f16_ok(a, w, c, m, n, k, f);
+  const bool forced = g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0;
+  if (gemm_few_ok(f, a, w, c, m, n, k) && (g_tune_gemm_few == 1 || !forced)) {
+    const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
+    const double engine = 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15);      // (gemm_few_tokens_by_engine)
+    const double cores = !cores_ok ? 1e30 : gemm_cut(d, f, m, n, k).waves == 4u ? 7.2 + mb / 4.0 : 12.0 + mb / 9.4;
+    if (g_tune_gemm_few == 1 || gemm_few_us(d, m, n) < std::min(engine, cores)) return GemmRoute::kFew;
+  }
+  if (cores_ok && (forced || !gemm_few_tokens_by_engine(d, f, m, n, k))) return GemmRoute::kCores;
+  return GemmRoute::kOther;
+}
+
 hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, uint64_t c, uint32_t m, uint32_t n,
                             uint32_t k, bool is_gemv, uint32_t flags = 0) {
   if (k % 256u != 0) return hipErrorInvalidValue;
@@ -593,16 +610,11 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   DeviceKernels* d = nullptr;
   hipError_t e = device_kernels(&d);
   if (e != hipSuccess) return e;
-  if (!is_gemv && gemm_few_ok(f, a, w, c, m, n, k)) {
-    // against the faster of the other two ways, by their fitted times (gemm_few_tokens_by_engine)
-    const double mb = double(n) * (k / 256u) * kSbBytes[f] / 1e6;
-    const double engine = 3.9 + mb / 5.7 + (m - 1u) * (mb / 5.8 + 0.15);
-    const double cores = !q4k_gemm_f16_ok(a, w, c, m, n, k, f) ? 1e30 : gemm_cut(*d, f, m, n, k).waves == 4u ? 7.2 + mb / 4.0 : 12.0 + mb / 9.4;
-    if (g_tune_gemm_few == 1 || gemm_few_us(*d, m, n) < std::min(engine, cores)) return launch_gemm_few(d, stream, a, w, c, m, n, k);
+  if (!is_gemv) {
+    const GemmRoute route = gemm_route(*d, f, a, w, c, m, n, k);
+    if (route == GemmRoute::kFew) return launch_gemm_few(d, stream, a, w, c, m, n, k);
+    if (route == GemmRoute::kCores) return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   }
-  if (!is_gemv && q4k_gemm_f16_ok(a, w, c, m, n, k, f) &&
-      (g_tune_gemm_ksplit > 0 || g_tune_gemm_waves > 0 || g_tune_gemm_tiles > 0 || !gemm_few_tokens_by_engine(*d, f, m, n, k)))
-    return launch_kq_gemm_f16(d, f, stream, a, w, c, m, n, k);
   const uint32_t grid_y = std::min<uint32_t>(m, 65535u);
   // GEMV parameter order is (y, w, x, k, n); GEMM is (a, b_quant, c, m, n, k)
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
@@ -1836,10 +1848,8 @@ trn_status trn_q4k_gemm_noalloc(trn_stream s, trn_dptr a, trn_dptr b, trn_dptr c
   hipStream_t stream = static_cast<hipStream_t>(s);
   DeviceKernels* d = nullptr;
   TRN_TRY(device_kernels(&d));
-  // the same choice of kernel as trn_q4k_gemm, so the same bits: the GEMV engine needs no scratch at all
-  if (!q4k_gemm_f16_ok(a, b, c, m, n, k) ||
-      (g_tune_gemm_ksplit == 0 && g_tune_gemm_waves == 0 && g_tune_gemm_tiles == 0 && gemm_few_tokens_by_engine(*d, Q4K, m, n, k)))
-    return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));
+  // the same choice of kernel as trn_q4k_gemm, so the same bits: only the f16 matrix-core form needs scratch at all
+  if (gemm_route(*d, Q4K, a, b, c, m, n, k) != GemmRoute::kCores) return st(launch_gemm_like(Q4K, stream, a, b, c, m, n, k, false));
   int dev = 0;
   TRN_TRY(hipGetDevice(&dev));
   size_t cap = 0;
