@@ -80,7 +80,7 @@ def traffic(fetch_dir: str, write_dir: str, kernel: str, json_out: str | None) -
               "yardstick": f"{COPY_KERNEL} over 256 MiB reads FETCH_SIZE {fetch[COPY_KERNEL][0]:.1f} KiB, WRITE_SIZE {write[COPY_KERNEL][0]:.1f} KiB",
               "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -d <dir> -- python3 bench.py --steps 2 --warmup 1 --pass-only"}
     try:
-        root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+        root = os.path.dirname(os.path.abspath(__file__))
         result["commit"] = subprocess.run(["git", "-C", root, "rev-parse", "--short", "HEAD"], capture_output=True, text=True,
                                           check=True).stdout.strip()
     except Exception:
