@@ -147,7 +147,12 @@ TRN_API trn_status trn_q5k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_d
 TRN_API trn_status trn_q6k_gemv(trn_stream stream, trn_dptr y, trn_dptr w, trn_dptr x, uint32_t k, uint32_t n);
 /* C[m x n] = A[m x k] . dequant(W[n x k])^T, c[row*n + col]; A, C f32 row-major.  The decode is the
  * GEMV-family one, so m = 1 equals the GEMV.  Replace QuantizeKernel::ggml / Q5KKernel / Q6KKernel
- * (quantize.rs:347-579, :640-866, :926-1121). */
+ * (quantize.rs:347-579, :640-866, :926-1121).  Which kernel takes a product is the library's choice by its shape (one
+ * token: the GEMV engine; Q4_K, two to four tokens, k <= 4096: the integer matrix cores where that is fastest; otherwise
+ * the f16 matrix cores, or for a few tokens against a small matrix the GEMV engine once per token); every one of them is
+ * within the 1e-5 relative L2 of fp64 and no worse than an f32 evaluation in the reference's order, but they are not
+ * bit-identical to each other.  An infinity or NaN among a token's activations makes that token's results non-finite
+ * (NaN where the reference's sum would give an infinity) and leaves the other tokens alone. */
 TRN_API trn_status trn_q4k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q5k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
 TRN_API trn_status trn_q6k_gemm(trn_stream stream, trn_dptr a, trn_dptr b_quant, trn_dptr c, uint32_t m, uint32_t n, uint32_t k);
@@ -309,14 +314,17 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * up to 4096; 16 or less keeps every launch on the kernel-argument form); "group_window": how far down the list a launch
  * looks for entries (0 = twice group_max); "group_waves": least waves per workgroup of a launch of up to sixteen entries (0 = 8,
  * or what its widest entry needs); "many_waves": waves per workgroup of a launch of more than sixteen entries (0 = 12);
- * "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch shares out its
- * workgroups (0 = 40).
+ * "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch of up to sixteen entries
+ * shares out its workgroups (0 = 40); "many_slab_weight": the same for a launch of more than sixteen (0 = 18);
+ * "many_item_kb": what every piece of an entry costs the workgroup that takes it, in KB of weights (0 = 64).
  * "gemv_stream_off": 1 = no matrix streams its rows through LDS (every GEMV loads its rows into registers straight from
  * memory; same bits); "gemv_stream_q6k": 1 = Q6_K matrices of up to 4096 columns stream too (slower, measured);
  * "gemv_stream_waves": waves per workgroup of a single streamed GEMV (0 = 4); "gemv_stream_min_rows": a single GEMV
  * streams when a wave gets at least this many rows (0 = 16); "gemv_stream_cost": percent of its bytes a streamed entry
  * counts for when a launch shares out its workgroups (0 = 95).
- * "gemm_mfma_off": 1 = the k-quant GEMMs never take the matrix-core form; "gemm_k_parts": into how many parts
+ * "gemm_few": the Q4_K product of two to four tokens on the integer matrix cores - 0 = where its estimated time is the
+ * lowest, 1 = wherever it can run, 2 = never.
+ * "gemm_mfma_off": 1 = the k-quant GEMMs never take the f16 matrix-core form; "gemm_k_parts": into how many parts
  * that form cuts K; "gemm_waves": 4, 8 or (Q4_K) 12 strips of 32 rows per workgroup; "gemm_tiles": 1 or 2 tiles of 16 tokens per
  * workgroup (0 for each of the three = chosen from the shape by an estimated time; any of them set also keeps a
  * product of a few tokens on the matrix cores);

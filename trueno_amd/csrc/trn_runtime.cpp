@@ -117,6 +117,8 @@ std::atomic<int> g_tune_stream_q6k{0};      // 1: Q6_K one-slab GEMVs stream thr
 std::atomic<int> g_tune_stream_cost{0};     // percent of its bytes a streamed entry counts for when a grouped launch shares out its workgroups (0: default)
 std::atomic<int> g_tune_stream_min_rows{0}; // a single GEMV streams when a wave gets at least this many rows (0: default)
 std::atomic<int> g_tune_many_waves{0};      // waves per workgroup of a launch of more than sixteen entries (0: 12)
+std::atomic<int> g_tune_many_item_kb{0};    // what a further piece of work costs a workgroup of such a launch, in KB of weights (0: default)
+std::atomic<int> g_tune_many_slab_weight{0};  // percent such a launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: default)
 std::atomic<int> g_tune_stream_waves{0};    // waves per workgroup of a single streamed GEMV (0: default)
 std::atomic<int> g_tune_gemm_few{0};        // the integer matrix-core kernel for two to four tokens: 0 by the rule, 1 wherever it can run, 2 never
 
@@ -753,6 +755,11 @@ constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (k
 constexpr double kSlabCost = 0.4;
 // what a streamed entry's bytes cost against an entry's on the register path (launch_gemv_group)
 constexpr double kStreamCost = 0.95;
+// launches of more than sixteen entries (plan_gemv_many): weight per further slab and what a piece of work costs a workgroup
+// (KB of weights).  The 7B pass: 730 / 718 / 704 / 702 / 702 / 708 / 711 us with 40 / 30 / 25 / 20 / 15 / 10 / 5 % per slab (with 40 %
+// the workgroups with the one-slab o matrices ended 35 us after those with the three-slab down matrices); the cost of a piece
+// made no difference between 1 and 128 KB, more was slower.
+constexpr double kManySlabCost = 0.18, kManyItemKb = 64.0;
 // Entries a launch takes by default: as many as the kernel holds, looked for among the next 32 of the list.  On the 7B
 // pass with activation buffers per layer: 8 entries (138 MB a launch, 30 launches) 879 us, 12 of the next 24 (21
 // launches) 820 us, 14 of 28 (18) 821 us, 16 of 32 (16 launches of 270 MB) 823 us; the launches of 12-16 entries run at
@@ -1574,37 +1581,46 @@ hipError_t plan_gemv_many(DeviceKernels* d, const trn_gemv_desc* descs, uint32_t
     const uint64_t limit = ring ? kStreamLdsLimit - ring : kFastLdsLimit;
     if (x_bytes + uint64_t(sw) * ug * 4u + kLdsScratch > limit) return hipErrorInvalidValue;
     const uint32_t max_rows = uint32_t(std::min<uint64_t>((limit - kLdsScratch - x_bytes) / (uint64_t(sw) * 4u) / ug * ug, 1u << 20));
-    const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
+    const double per_slab = g_tune_many_slab_weight > 0 ? int(g_tune_many_slab_weight) / 100.0 : kManySlabCost;
     const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
     const double cost = double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (sw - 1u)) * (ring ? stream_cost : 1.0);
     ent[i] = {cost, ring, sw, max_rows, x_bytes};
     total += cost;
   }
-  const double part = total / G;
+  // Every piece of an entry that a workgroup takes costs it a start of its own (the vector staged, the first batches on
+  // their way, the last ones summed with nothing behind them): item_cost, in the axis's bytes.  The workgroups are filled
+  // one after the other up to their share of the axis so far, so that what one leaves over the next ones get.
+  const double item_cost = (g_tune_many_item_kb > 0 ? double(int(g_tune_many_item_kb)) : kManyItemKb) * 1024.0;
+  const double part = (total + item_cost * (double(len) + double(G))) / G;
   std::vector<std::vector<uint32_t>> items_of(G);      // per workgroup: (entry, row0, rows) triples
   uint32_t lds = 0;
-  double start = 0.0;
-  for (uint32_t i = 0; i < len; ++i) {
-    const trn_gemv_desc& e = descs[i];
-    const double end = start + ent[i].cost;
-    const uint32_t w0 = std::min(G - 1u, uint32_t(start / part)), w1 = std::min(G - 1u, uint32_t(std::max(start, end - 1e-9 * part) / part));
-    uint32_t row = 0;
-    for (uint32_t w = w0; w <= w1 && row < e.n; ++w) {
-      uint32_t upto = e.n;
-      if (w < w1) {
-        const double frac = (double(w + 1u) * part - start) / ent[i].cost;
-        upto = uint32_t(std::min<double>(double(e.n), std::max(0.0, frac * double(e.n)) + 0.5)) / ug * ug;
-        if (upto < row + 32u) continue;                 // too small a piece at the entry's start: the next workgroup takes it
-        if (e.n - upto < 32u) upto = e.n;               // ... at its end: this one takes it
+  double assigned = 0.0;
+  uint32_t i = 0, row = 0;
+  for (uint32_t w = 0; w < G && i < len; ++w) {
+    const bool last = w + 1u == G;
+    while (i < len) {
+      const trn_gemv_desc& e = descs[i];
+      const double per_row = ent[i].cost / double(e.n);
+      const uint32_t left = e.n - row;
+      uint32_t take = left;
+      if (!last) {
+        const double budget = double(w + 1u) * part - assigned - item_cost;
+        take = budget <= 0.0 ? 0u : uint32_t(std::min<double>(double(left), budget / per_row + 0.5)) / ug * ug;
+        if (take < 32u && !items_of[w].empty()) break;      // too small a piece: the next workgroup takes it
+        take = std::max(take, std::min(left, 32u));          // (a workgroup with nothing yet takes something)
+        if (left - take < 32u) take = left;                  // a small rest at the entry's end stays with this one
       }
-      while (row < upto) {
-        const uint32_t rows = std::min((upto - row + ug - 1u) / ug * ug, ent[i].max_rows);
-        items_of[w].insert(items_of[w].end(), {i, row, rows});
+      for (uint32_t done = 0; done < take;) {
+        const uint32_t rows = std::min((take - done + ug - 1u) / ug * ug, ent[i].max_rows);
+        items_of[w].insert(items_of[w].end(), {i, row + done, rows});
         lds = std::max<uint32_t>(lds, uint32_t(ent[i].x_bytes + uint64_t(ent[i].sw) * rows * 4u + kLdsScratch + ent[i].ring));
-        row += rows;
+        done += rows;
       }
+      assigned += item_cost + per_row * take;
+      row += take;
+      if (row >= e.n) { ++i; row = 0; }
+      if (!last && assigned >= double(w + 1u) * part - item_cost) break;
     }
-    start = end;
   }
   size_t n_items = 0;
   for (const auto& v : items_of) n_items += v.size() / 3u;
@@ -1975,6 +1991,8 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemv_stream_off")) { g_tune_stream_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_waves")) { g_tune_stream_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "many_waves")) { g_tune_many_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "many_item_kb")) { g_tune_many_item_kb = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "many_slab_weight")) { g_tune_many_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_q6k")) { g_tune_stream_q6k = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_cost")) { g_tune_stream_cost = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_min_rows")) { g_tune_stream_min_rows = value; return TRN_SUCCESS; }
