@@ -8,8 +8,12 @@
 // and an end (token conversion, the sum over the parts of K across workgroups) of 8 us.  Here the weights are read once
 // for all tokens, the multiply-adds run on the matrix cores, and what is left to the vector unit is one AND per four
 // weights and a handful of instructions per (row, sub-block, token).  Measured on MI355X (14336 x 4096, cold weights):
-// 11.2 us for two tokens and 13.1 us for four, against 14.8 us for either through the f16 form.  More tokens do not pay:
-// every workgroup needs the digits of every token, and with eight that start alone takes 6 us.
+// 10.6 us for two tokens and 13.1 us for four, against 14.8 us for either through the f16 form.  More tokens do not pay:
+// every workgroup needs the digits of every token, and with eight that start alone takes 6 us.  Time stamps inside
+// the kernel (four tokens, two tiles per workgroup): activations there at 0.8 us, digits in the registers at 4.3-6.5 us
+// (the copy instructions of a tile take a wave 0.5 us to issue and block it once about 64 KB per CU are in flight, so
+// copies requested early delay the conversion behind them), first tile staged at 7.5 us, 1.4 us to multiply a tile,
+// second tile staged at 10 us, end at 12.3 us.
 //
 // Arithmetic.  For a token t and a run of 256 activations (a super-block's columns) the activations are brought to
 // integers X = rint(x * 2^e) with |X| <= 2^30 (e from the run's largest magnitude) and cut into four signed digits of
@@ -33,8 +37,10 @@
 // Wave w multiplies the super-blocks 2 w and 2 w + 1 of a tile's rows (its 64 registers of digits cover those 512
 // columns for the whole launch): it takes its part of a landed tile into registers, and when every wave has, the
 // buffer is given to the tile after next - two tiles are on their way while one is multiplied.  The eight waves' shares
-// of a tile meet in LDS and are added in wave order.  The digits are made once per workgroup and reach the waves through
-// the second tile buffer, while the first tile is already on its way.
+// of a tile meet in LDS (two areas in turn) and are added in wave order while the next tile is multiplied.  The digits
+// are made once per workgroup, two tokens at a time, and reach the waves through the upper half of the second tile
+// buffer, while the first tile and the lower half of the second are already on their way.  No barrier of the kernel
+// waits for copies in flight (wg_barrier).
 #pragma once
 #include "kquant_common.hip.h"
 
@@ -47,14 +53,16 @@ constexpr u32 kWaves = 8;
 constexpr u32 kTileRows = 32;
 constexpr u32 kRowPad = 32;                     // LDS bytes between the end of a row and the start of the next
 __host__ __device__ constexpr u32 row_stride(u32 nsb) { return nsb * 144u + kRowPad; }
-// dynamic LDS: two tile buffers (which hold the digits first), the waves' partial results, the sub-block sums and scales
 __host__ __device__ constexpr u32 tile_bytes(u32 nsb) { return kTileRows * row_stride(nsb); }
+// dynamic LDS: two tile buffers (the upper half of the second holds the digits first), two areas for the waves' partial
+// results, the sub-block sums and scales of the tokens
 __host__ __device__ constexpr u32 lds_bytes(u32 nsb, u32 ntok) {
-  return 2u * tile_bytes(nsb) + kWaves * kTileRows * ntok * 4u + ntok * nsb * 9u * 4u;
+  return 2u * tile_bytes(nsb) + 2u * kWaves * kTileRows * ntok * 4u + ntok * nsb * 9u * 4u;
 }
-// the digits on their way to the registers: per sub-block and half of it, 4 ntok operand rows of 16 bytes
-__host__ __device__ constexpr u32 digit_bytes(u32 nsb, u32 ntok) { return nsb * 8u * 2u * 4u * ntok * 16u; }
-static_assert(digit_bytes(16, 4) <= tile_bytes(16) && digit_bytes(1, 4) <= tile_bytes(1), "the digits of four tokens fit one tile buffer");
+// the digits of two tokens on their way to the registers: per half sub-block eight operand rows of 16 bytes
+__host__ __device__ constexpr u32 digit_bytes(u32 nsb) { return nsb * 16u * 8u * 16u; }
+static_assert(digit_bytes(16) <= tile_bytes(16) / 2u && digit_bytes(1) <= tile_bytes(1) / 2u, "two tokens' digits fit half a tile buffer");
+static_assert(lds_bytes(16, 4) <= 160u * 1024u, "LDS of a CU");
 
 __device__ __forceinline__ void lds_r128(u32x4& v, u32 addr) { asm volatile("ds_read_b128 %0, %1" : "=&v"(v) : "v"(addr) : "memory"); }
 __device__ __forceinline__ void lds_r32(u32& v, u32 addr) { asm volatile("ds_read_b32 %0, %1" : "=&v"(v) : "v"(addr) : "memory"); }
@@ -73,7 +81,10 @@ __device__ __forceinline__ u32 row_max_u32(u32 v) {
   v = max(v, static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, true)));
   return v;
 }
-
+// Workgroup barrier over the LDS accesses only (all of them are written in asm here).  __syncthreads() would also wait
+// for every copy into LDS that is in flight - the compiler places s_waitcnt vmcnt(0) in front of its barrier - which is
+// the one thing the order of the copies is there to avoid.
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 // at most n of this wave's vector-memory operations outstanding (n <= 14 here)
 __device__ __forceinline__ void wait_vm(u32 n) {
   switch (n) {
@@ -100,16 +111,18 @@ __device__ __forceinline__ void store_f32(float* p, float v) {
 template <int NTOK>
 __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint8_t* __restrict__ w, float* __restrict__ c, u32 m, u32 n,
                                          u32 k, u32 row0, u32 rows, u32 lds) {
-  static_assert(NTOK == 2 || NTOK == 4, "two or four tokens: the digits of more do not fit beside the first tile");
+  static_assert(NTOK == 2 || NTOK == 4, "two or four tokens");
   constexpr int NA = NTOK / 2;                      // tokens per lane: 2 a + l / 32, a < NA
+  constexpr int PHASES = NTOK / 2;                  // the digits are made two tokens at a time
   const u32 tid = threadIdx.x, lane = tid & 63u;
   const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(tid >> 6)));
   const u32 nsb = k >> 8;                           // 1 .. 16
   const u32 row_bytes = nsb * 144u, rs = row_stride(nsb), tb = tile_bytes(nsb);
   const u32 lds_tiles = lds;
-  const u32 lds_red = lds + 2u * tb;
-  const u32 lds_dig = lds_tiles + tb;                                  // the digits' way to the registers: the second tile buffer
-  const u32 lds_sx = lds_red + kWaves * kTileRows * NTOK * 4u;         // [token][sub-block of the row] f32 sums of X
+  const u32 lds_dig = lds_tiles + tb + 16u * rs;                       // the digits' way to the registers: rows 16 .. 31 of the second buffer
+  const u32 red_bytes = kWaves * kTileRows * NTOK * 4u;
+  const u32 lds_red = lds + 2u * tb;                                   // [tile parity][wave][row][token] f32
+  const u32 lds_sx = lds_red + 2u * red_bytes;                         // [token][sub-block of the row] f32 sums of X
   const u32 lds_fs = lds_sx + NTOK * nsb * 8u * 4u;                    // [token][super-block] f32: 2^-e
   const u32 col = lane & 31u, g = lane >> 5;
 
@@ -132,108 +145,136 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
     }
   };
   const u32 per_tile = 4u * (full + 1u);             // copies a wave issues per tile: 4, 8 or 12
+
   // ---- the digits: 16 lanes convert one (token, super-block) run, 16 values each ------------------------------------
-  // 16 NTOK nsb tasks over 512 threads (nsb <= 16): the activations of every round are asked for first
-  constexpr int ROUNDS = NTOK / 2;
-  const u32 tasks = NTOK * nsb * 16u;
-  f32x4 xall[ROUNDS][4];
+  // thread = (token of the pair tid / 256, half sub-block tid % 256 = 16 sb + q16); phase p converts the tokens 2 p, 2 p + 1.
+  // The activations of every phase are asked for first.
+  const u32 tt = tid >> 8, half_mine = tid & 255u;
+  const bool task = half_mine < nsb * 16u;
+  const u32 sb_mine = half_mine >> 4, q16 = half_mine & 15u;
+  f32x4 xall[PHASES][4];
 #pragma unroll
-  for (int rd = 0; rd < ROUNDS; ++rd) {
-    const u32 task = tid + 64u * kWaves * rd, run = task >> 4;
-    const u32 t = run / nsb, sb = run - t * nsb;
-    if (task < tasks && t < m) {
-      const f32x4* src = reinterpret_cast<const f32x4*>(a + static_cast<size_t>(t) * k + sb * 256u + (task & 15u) * 16u);
+  for (int ph = 0; ph < PHASES; ++ph) {
+    const u32 t = tt + 2u * ph;
+    if (task && t < m) {
+      const f32x4* src = reinterpret_cast<const f32x4*>(a + static_cast<size_t>(t) * k + half_mine * 16u);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xall[rd][i] = src[i];
+      for (int i = 0; i < 4; ++i) xall[ph][i] = src[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xall[rd][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int i = 0; i < 4; ++i) xall[ph][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
   }
   // The first tile sets out before the digits are made, but behind the activations: loads return in the order they
-  // were issued, and the compiler waits for its loads as if the copies were not there.
+  // were issued, and the compiler waits for its loads as if the copies were not there.  The second tile's lower half
+  // (the waves 0 .. 3) follows at once; its upper half is where the digits pass through.
 #pragma unroll
-  for (int rd = 0; rd < ROUNDS; ++rd) asm volatile("" : "+v"(xall[rd][0]), "+v"(xall[rd][1]), "+v"(xall[rd][2]), "+v"(xall[rd][3])::"memory");
+  for (int ph = 0; ph < PHASES; ++ph) asm volatile("" : "+v"(xall[ph][0]), "+v"(xall[ph][1]), "+v"(xall[ph][2]), "+v"(xall[ph][3])::"memory");
   issue(0u);
-#pragma unroll
-  for (int rd = 0; rd < ROUNDS; ++rd) {
-    const u32 task = tid + 64u * kWaves * rd;
-    if (task >= tasks) break;
-    const u32 run = task >> 4, q16 = task & 15u;
-    const u32 t = run / nsb, sb = run - t * nsb;
-    const f32x4* xv = xall[rd];
-    u32 amax = 0u;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      amax = max(max(amax, __float_as_uint(xv[i].x) & 0x7FFFFFFFu),
-                 max(max(__float_as_uint(xv[i].y) & 0x7FFFFFFFu, __float_as_uint(xv[i].z) & 0x7FFFFFFFu), __float_as_uint(xv[i].w) & 0x7FFFFFFFu));
-    amax = row_max_u32(amax);
-    u32 eb = amax >> 23;                             // biased exponent of the run's largest magnitude: |x| < 2^(eb - 126)
-    const bool finite = eb != 255u;
-    eb = eb < 30u ? 30u : eb;                        // keeps both powers of two normal numbers
-    const float up = __uint_as_float((283u - eb) << 23);       // 2^(156 - eb): |x| * up < 2^30
-    // X + 0x808080 has the bytes D + 128 (D3 as it is): the xor makes signed bytes of them.  Then the 4 x 4 bytes of four
-    // values are transposed: plane[d] word v = digit d of the values 4 v .. 4 v + 3.
-    u32x4 plane[4];
-    int dsum[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float xs[4] = {xv[v].x, xv[v].y, xv[v].z, xv[v].w};
-      u32 z[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) z[i] = (static_cast<u32>(static_cast<int>(__builtin_rintf(xs[i] * up))) + 0x00808080u) ^ 0x00808080u;
-      const u32 t0 = __builtin_amdgcn_perm(z[1], z[0], 0x05010400u), t1 = __builtin_amdgcn_perm(z[1], z[0], 0x07030602u);
-      const u32 u0 = __builtin_amdgcn_perm(z[3], z[2], 0x05010400u), u1 = __builtin_amdgcn_perm(z[3], z[2], 0x07030602u);
-      plane[0][v] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
-      plane[1][v] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
-      plane[2][v] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
-      plane[3][v] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
-#pragma unroll
-      for (int d = 0; d < 4; ++d) dsum[d] = __builtin_amdgcn_sdot4(static_cast<int>(plane[d][v]), 0x01010101, dsum[d], false);
-    }
-    // consumer: sub-block sb * 8 + q16 / 2 of the row, half q16 % 2, operand row 4 t + d
-    const u32 dst = lds_dig + (((sb * 8u + (q16 >> 1)) * 2u + (q16 & 1u)) * (4u * NTOK) + 4u * t) * 16u;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) lds_w128(dst + 16u * d, plane[d]);
-    // SX of the sub-block: the digits' sums over its 32 values (with the neighbour's half), joined in f32
-#pragma unroll
-    for (int d = 0; d < 4; ++d) dsum[d] += __builtin_amdgcn_update_dpp(0, dsum[d], 0xB1, 0xF, 0xF, true);
-    const float sx = fmaf(static_cast<float>(dsum[3]), 16777216.0f, fmaf(static_cast<float>(dsum[2]), 65536.0f,
-                          fmaf(static_cast<float>(dsum[1]), 256.0f, static_cast<float>(dsum[0]))));
-    if ((q16 & 1u) == 0u) lds_w32(lds_sx + (t * nsb * 8u + sb * 8u + (q16 >> 1)) * 4u, __float_as_uint(sx));
-    if (q16 == 0u) lds_w32(lds_fs + (t * nsb + sb) * 4u, finite ? (eb - 29u) << 23 : 0x7FC00000u);      // 2^(eb - 156) = 1 / up
-  }
-  lds_wait();
-  __syncthreads();
-  // this wave's digits: sub-blocks 0 .. 15 of its two super-blocks, operand row col (= 4 t + d) and half g of the sub-block
+  if (wave < 4u && tiles > 1u) issue(1u);
   i32x4 dig[16];
-  {
-    u32x4 raw[16];
-    const u32 from = lds_dig + (((wave * 16u) * 2u + g) * (4u * NTOK) + (col < 4u * NTOK ? col : 0u)) * 16u;
 #pragma unroll
-    for (int js = 0; js < 16; ++js)
-      if (wave * 16u + js < nsb * 8u) lds_r128(raw[js], from + js * (2u * 4u * NTOK * 16u)); else raw[js] = u32x4{0u, 0u, 0u, 0u};
-    lds_wait();
+  for (int js = 0; js < 16; ++js) dig[js] = i32x4{0, 0, 0, 0};
 #pragma unroll
-    for (int js = 0; js < 16; ++js) {
-      asm volatile("" : "+v"(raw[js]));
-      if (col >= 4u * NTOK) raw[js] = u32x4{0u, 0u, 0u, 0u};      // rows of tokens the kernel is not built for
-      dig[js] = __builtin_bit_cast(i32x4, raw[js]);
+  for (int ph = 0; ph < PHASES; ++ph) {
+    if (task) {
+      const u32 t = tt + 2u * ph;
+      const f32x4* xv = xall[ph];
+      u32 amax = 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        amax = max(max(amax, __float_as_uint(xv[i].x) & 0x7FFFFFFFu),
+                   max(max(__float_as_uint(xv[i].y) & 0x7FFFFFFFu, __float_as_uint(xv[i].z) & 0x7FFFFFFFu), __float_as_uint(xv[i].w) & 0x7FFFFFFFu));
+      amax = row_max_u32(amax);
+      u32 eb = amax >> 23;                           // biased exponent of the run's largest magnitude: |x| < 2^(eb - 126)
+      const bool finite = eb != 255u;
+      eb = eb < 30u ? 30u : eb;                      // keeps both powers of two normal numbers
+      const float up = __uint_as_float((283u - eb) << 23);       // 2^(156 - eb): |x| * up < 2^30
+      // X + 0x808080 has the bytes D + 128 (D3 as it is): the xor makes signed bytes of them.  Then the 4 x 4 bytes of four
+      // values are transposed: plane[d] word v = digit d of the values 4 v .. 4 v + 3.
+      u32x4 plane[4];
+      int dsum[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float xs[4] = {xv[v].x, xv[v].y, xv[v].z, xv[v].w};
+        u32 z[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) z[i] = (static_cast<u32>(static_cast<int>(__builtin_rintf(xs[i] * up))) + 0x00808080u) ^ 0x00808080u;
+        const u32 t0 = __builtin_amdgcn_perm(z[1], z[0], 0x05010400u), t1 = __builtin_amdgcn_perm(z[1], z[0], 0x07030602u);
+        const u32 u0 = __builtin_amdgcn_perm(z[3], z[2], 0x05010400u), u1 = __builtin_amdgcn_perm(z[3], z[2], 0x07030602u);
+        plane[0][v] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
+        plane[1][v] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
+        plane[2][v] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
+        plane[3][v] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) dsum[d] = __builtin_amdgcn_sdot4(static_cast<int>(plane[d][v]), 0x01010101, dsum[d], false);
+      }
+      // Consumer: half sub-block `half_mine` of the row, operand row 4 (token of the pair) + d of the eight of this phase.
+      // The eight rows of a half sub-block lie 16 bytes apart in an order rotated by the half sub-block's number, so that
+      // the sixteen lanes that write one row of sixteen neighbouring half sub-blocks do not all hit the same banks.
+      const u32 dst = lds_dig + half_mine * 128u;
+#pragma unroll
+      for (u32 d = 0; d < 4u; ++d) lds_w128(dst + (((4u * tt + d) ^ half_mine) & 7u) * 16u, plane[d]);
+      // SX of the sub-block: the digits' sums over its 32 values (with the neighbour's half), joined in f32
+#pragma unroll
+      for (int d = 0; d < 4; ++d) dsum[d] += __builtin_amdgcn_update_dpp(0, dsum[d], 0xB1, 0xF, 0xF, true);
+      const float sx = fmaf(static_cast<float>(dsum[3]), 16777216.0f, fmaf(static_cast<float>(dsum[2]), 65536.0f,
+                            fmaf(static_cast<float>(dsum[1]), 256.0f, static_cast<float>(dsum[0]))));
+      if ((q16 & 1u) == 0u) lds_w32(lds_sx + (t * nsb * 8u + sb_mine * 8u + (q16 >> 1)) * 4u, __float_as_uint(sx));
+      if (q16 == 0u) lds_w32(lds_fs + (t * nsb + sb_mine) * 4u, finite ? (eb - 29u) << 23 : 0x7FC00000u);      // 2^(eb - 156) = 1 / up
     }
+    wg_barrier();
+    // this wave's digits of this phase's tokens: sub-blocks 0 .. 15 of its two super-blocks, operand row col (= 4 t + d)
+    // and half g of the sub-block; operand rows of tokens the kernel is not built for stay zero
+    if ((col >> 3) == static_cast<u32>(ph)) {
+      u32x4 raw[16];
+#pragma unroll
+      for (u32 js = 0; js < 16u; ++js) {
+        const u32 half = (wave * 16u + js) * 2u + g;
+        if (wave * 16u + js < nsb * 8u) lds_r128(raw[js], lds_dig + half * 128u + (((col & 7u) ^ half) & 7u) * 16u);
+        else raw[js] = u32x4{0u, 0u, 0u, 0u};
+      }
+      lds_wait();
+#pragma unroll
+      for (int js = 0; js < 16; ++js) {
+        asm volatile("" : "+v"(raw[js]));
+        dig[js] = __builtin_bit_cast(i32x4, raw[js]);
+      }
+    }
+    wg_barrier();                                    // the digits are read: the next phase's, or the tile's rows, may come
   }
-  __syncthreads();                                   // everybody has its digits: the buffers may take tiles
-  if (tiles > 1u) issue(1u);
+  if (wave >= 4u && tiles > 1u) issue(1u);
 
   // ---- tiles --------------------------------------------------------------------------------------------------------
-  // Results leave through the waves that hold the threads 0 .. 32 NTOK - 1: ONE store per tile and wave, issued by every
-  // lane (lanes without a result of their own repeat a neighbour's), so that the number of this wave's memory operations
-  // behind a tile's copies is known: the next tile's copies, and the stores of the two tiles before.
-  const bool stores = wave * 64u < kTileRows * NTOK;
+  // A tile's results leave while the next tile is multiplied: every wave adds up its share of them (4 NTOK of the
+  // 32 NTOK) and issues ONE store per tile, by every lane (lanes without a result of their own repeat a neighbour's),
+  // so that the number of this wave's memory operations behind a tile's copies is known: the next tile's copies and the
+  // stores issued since.
   const bool active0 = 2u * wave < nsb, active1 = 2u * wave + 1u < nsb;
+  auto reduce_store = [&](u32 tile) {
+    const u32 o = wave * (4u * NTOK) + (lane & (4u * NTOK - 1u));
+    const u32 valid = min(kTileRows, rows - tile * kTileRows);      // rows of this tile that exist (>= 1)
+    u32 r = o / NTOK, t = o & (NTOK - 1u);
+    r = r < valid ? r : valid - 1u;
+    t = t < m ? t : m - 1u;
+    const u32 from = lds_red + (tile & 1u) * red_bytes + (r * NTOK + t) * 4u;
+    u32 part[kWaves];
+#pragma unroll
+    for (u32 wv = 0; wv < kWaves; ++wv) lds_r32(part[wv], from + wv * kTileRows * NTOK * 4u);
+    lds_wait();
+    float sum = 0.0f;
+#pragma unroll
+    for (u32 wv = 0; wv < kWaves; ++wv) {
+      asm volatile("" : "+v"(part[wv]));
+      if (2u * wv < nsb) sum += __uint_as_float(part[wv]);
+    }
+    store_f32(c + static_cast<size_t>(t) * n + (row0 + tile * kTileRows + r), sum);
+  };
   for (u32 tile = 0; tile < tiles; ++tile) {
-    // tile `tile` has landed when no more of this wave's operations are outstanding than were issued behind its copies
-    wait_vm(tile + 1u < tiles ? per_tile + (stores ? (tile < 2u ? tile : 2u) : 0u) : 0u);
-    __syncthreads();
+    // tile `tile` has landed when no more of this wave's operations are outstanding than were issued behind its copies:
+    // the next tile's copies, and the stores of the tiles tile - 3 and tile - 2 (issued in the two rounds before)
+    wait_vm(tile + 1u < tiles ? per_tile + (tile >= 3u ? 2u : tile >= 2u ? 1u : 0u) : 0u);
+    wg_barrier();
     // this wave's part of the tile goes to registers, so that the buffer can take the tile after next while this one is
     // multiplied: two tiles on their way at any time
     const u32 rowp = lds_tiles + (tile & 1u) * tb + col * rs + 2u * wave * 144u;
@@ -250,8 +291,9 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
     for (u32 sbi = 0; sbi < 2u; ++sbi)
       if (sbi == 0u ? active0 : active1)
         asm volatile("" : "+v"(hdr2[sbi]), "+v"(pc2[sbi][0]), "+v"(pc2[sbi][1]), "+v"(pc2[sbi][2]), "+v"(pc2[sbi][3]));
-    __syncthreads();                                 // every wave has its part: the buffer is free
+    wg_barrier();                                    // every wave has its part (and wrote its share of the tile before): the buffer is free
     if (tile + 2u < tiles) issue(tile + 2u);
+    if (tile > 0u) reduce_store(tile - 1u);
     float y[NA];
 #pragma unroll
     for (int aa = 0; aa < NA; ++aa) y[aa] = 0.0f;
@@ -266,10 +308,9 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
 #pragma unroll
       for (int aa = 0; aa < NA; ++aa) {
         const u32 t = 2u * aa + g;
-        const u32 tt = t < static_cast<u32>(NTOK) ? t : 0u;
-        lds_r128(sxa[aa][0], lds_sx + (tt * nsb * 8u + sb * 8u) * 4u);
-        lds_r128(sxa[aa][1], lds_sx + (tt * nsb * 8u + sb * 8u + 4u) * 4u);
-        lds_r32(fsa[aa], lds_fs + (tt * nsb + sb) * 4u);
+        lds_r128(sxa[aa][0], lds_sx + (t * nsb * 8u + sb * 8u) * 4u);
+        lds_r128(sxa[aa][1], lds_sx + (t * nsb * 8u + sb * 8u + 4u) * 4u);
+        lds_r32(fsa[aa], lds_fs + (t * nsb + sb) * 4u);
       }
       lds_wait();
 #pragma unroll
@@ -313,34 +354,14 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
         y[aa] += fmaf(-(dmin * f), Q[aa], (d * f) * P[aa]);
       }
     }
-    // the waves' shares of the tile meet in LDS: red[wave][row][token]
+    // the waves' shares of the tile meet in LDS: red[tile parity][wave][row][token]; they are added up behind the next
+    // tile's barriers (or behind the loop), which every wave reaches after these writes
 #pragma unroll
-    for (int aa = 0; aa < NA; ++aa) {
-      const u32 t = 2u * aa + g;
-      if (t < static_cast<u32>(NTOK)) lds_w32(lds_red + ((wave * kTileRows + col) * NTOK + t) * 4u, __float_as_uint(y[aa]));
-    }
-    lds_wait();
-    __syncthreads();                                 // every wave has written its share
-    if (stores) {
-      const u32 o = tid < kTileRows * NTOK ? tid : kTileRows * NTOK - 1u;
-      const u32 valid = min(kTileRows, rows - tile * kTileRows);      // rows of this tile that exist (>= 1)
-      u32 r = o / NTOK, t = o - r * NTOK;
-      r = r < valid ? r : valid - 1u;
-      t = t < m ? t : m - 1u;
-      u32 part[kWaves];
-#pragma unroll
-      for (u32 wv = 0; wv < kWaves; ++wv) lds_r32(part[wv], lds_red + ((wv * kTileRows + r) * NTOK + t) * 4u);
-      lds_wait();
-      float sum = 0.0f;
-#pragma unroll
-      for (u32 wv = 0; wv < kWaves; ++wv) {
-        asm volatile("" : "+v"(part[wv]));
-        if (2u * wv < nsb) sum += __uint_as_float(part[wv]);
-      }
-      store_f32(c + static_cast<size_t>(t) * n + (row0 + tile * kTileRows + r), sum);
-    }
-    // (the next tile's shares are written behind its barriers at the top, which every thread reaches after these reads)
+    for (int aa = 0; aa < NA; ++aa)
+      lds_w32(lds_red + (tile & 1u) * red_bytes + ((wave * kTileRows + col) * NTOK + 2u * aa + g) * 4u, __float_as_uint(y[aa]));
   }
+  wg_barrier();
+  reduce_store(tiles - 1u);
 }
 
 }  // namespace few_i8
