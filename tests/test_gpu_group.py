@@ -166,6 +166,28 @@ def test_many_entries_in_one_launch(gpu, seed):
         assert kq.rel_l2(got[dst], ref) <= TOL, (seed, dst, fmt, n, k)
 
 
+@pytest.mark.parametrize("item_kb,slab_weight", [(4000, 90), (1, 1)])
+def test_many_entries_whatever_the_weights_of_the_cut(gpu, item_kb, slab_weight):
+    """How a large launch shares out its workgroups (the cost of a piece of work, the weight of a further slab) decides
+    which workgroup takes which rows and nothing else: with a piece at 4 MB (most workgroups then get too much and the last
+    ones nothing) or at nothing the results are the bits of one launch per entry."""
+    rng = np.random.default_rng(7)
+    specs = [(("q4k", "q5k", "q6k")[int(rng.integers(3))], int(rng.choice((1, 31, 33, 640, 2817))), int(rng.choice((256, 4096, 8192, 11008))),
+              "x", f"y{i}", int(rng.integers(2))) for i in range(40)]
+    sep, _ = _run(gpu, specs, 11008, 1)
+    try:
+        _tune("many_item_kb", item_kb)
+        _tune("many_slab_weight", slab_weight)
+        plan = []
+        got, _ = _run(gpu, specs, 11008, 0, plan)
+    finally:
+        _tune("many_item_kb", 0)
+        _tune("many_slab_weight", 0)
+    assert max(plan) == 0, plan
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), name
+
+
 def test_many_entries_plan_is_reused_and_replaced(gpu):
     """The cut of a list and its device tables are kept per stream for as long as the same list comes again; another list
     replaces them.  Two lists issued alternately on one stream, each twice in a row: always the bits of one launch per entry."""

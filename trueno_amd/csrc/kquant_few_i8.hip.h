@@ -8,12 +8,11 @@
 // and an end (token conversion, the sum over the parts of K across workgroups) of 8 us.  Here the weights are read once
 // for all tokens, the multiply-adds run on the matrix cores, and what is left to the vector unit is one AND per four
 // weights and a handful of instructions per (row, sub-block, token).  Measured on MI355X (14336 x 4096, cold weights):
-// 10.6 us for two tokens and 13.1 us for four, against 14.8 us for either through the f16 form.  More tokens do not pay:
+// 10.3 us for two tokens and 12.3 us for four, against 14.8 us for either through the f16 form.  More tokens do not pay:
 // every workgroup needs the digits of every token, and with eight that start alone takes 6 us.  Time stamps inside
-// the kernel (four tokens, two tiles per workgroup): activations there at 0.8 us, digits in the registers at 4.3-6.5 us
-// (the copy instructions of a tile take a wave 0.5 us to issue and block it once about 64 KB per CU are in flight, so
-// copies requested early delay the conversion behind them), first tile staged at 7.5 us, 1.4 us to multiply a tile,
-// second tile staged at 10 us, end at 12.3 us.
+// the kernel (four tokens, two tiles per workgroup): activations there at 0.8 us, first copies asked for at 1.1 us, digits
+// in the registers at 4.9 us, first tile staged at 6.5 us (all 224 workgroups ask for their first 75 KB at once: 16.8 MB),
+// 1.4 us to multiply a tile, second tile staged at 8.9 us, end at 11.3 us.
 //
 // Arithmetic.  For a token t and a run of 256 activations (a super-block's columns) the activations are brought to
 // integers X = rint(x * 2^e) with |X| <= 2^30 (e from the run's largest magnitude) and cut into four signed digits of
@@ -131,10 +130,11 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
   const u32 full = row_bytes >> 10, rem16 = (row_bytes & 1023u) >> 4;        // whole KB of a row, 16-byte pieces behind them
   // wave w copies rows 4 w .. 4 w + 3 of a tile: per row `full` instructions of 64 pieces and one of rem16 pieces
   // (144 nsb is never a multiple of 1024 for nsb <= 16: every row has the short copy)
-  auto issue = [&](u32 tile) {
+  // (the rows rb .. re - 1 of its four: a wave that issues more copies than the CU can have in flight - about 64 KB - stands
+  // still until earlier ones have landed, so the copies of a tile are issued in slices between slices of other work)
+  auto issue_rows = [&](u32 tile, u32 rb, u32 re) {
     const u32 buf = lds_tiles + (tile & 1u) * tb;
-#pragma unroll
-    for (u32 r = 0; r < 4u; ++r) {
+    for (u32 r = rb; r < re; ++r) {
       const u32 tr = 4u * wave + r;
       u32 row = row0 + tile * kTileRows + tr;
       row = row < n ? row : n - 1u;                  // rows behind the matrix re-read its last row: never stored
@@ -144,6 +144,7 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
       if (lane < rem16) dma16(src + 1024u * full, dst + 1024u * full);
     }
   };
+  auto issue = [&](u32 tile) { issue_rows(tile, 0u, 4u); };
   const u32 per_tile = 4u * (full + 1u);             // copies a wave issues per tile: 4, 8 or 12
 
   // ---- the digits: 16 lanes convert one (token, super-block) run, 16 values each ------------------------------------
@@ -170,8 +171,7 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
   // (the waves 0 .. 3) follows at once; its upper half is where the digits pass through.
 #pragma unroll
   for (int ph = 0; ph < PHASES; ++ph) asm volatile("" : "+v"(xall[ph][0]), "+v"(xall[ph][1]), "+v"(xall[ph][2]), "+v"(xall[ph][3])::"memory");
-  issue(0u);
-  if (wave < 4u && tiles > 1u) issue(1u);
+  issue_rows(0u, 0u, 2u);
   i32x4 dig[16];
 #pragma unroll
   for (int js = 0; js < 16; ++js) dig[js] = i32x4{0, 0, 0, 0};
@@ -223,6 +223,10 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
       if ((q16 & 1u) == 0u) lds_w32(lds_sx + (t * nsb * 8u + sb_mine * 8u + (q16 >> 1)) * 4u, __float_as_uint(sx));
       if (q16 == 0u) lds_w32(lds_fs + (t * nsb + sb_mine) * 4u, finite ? (eb - 29u) << 23 : 0x7FC00000u);      // 2^(eb - 156) = 1 / up
     }
+    // the next slice of copies: the rest of the first tile, then the lower half of the second (rows 0 .. 15: the waves
+    // 0 .. 3), whose upper half is where the digits pass through
+    if (ph == 0) issue_rows(0u, 2u, 4u);
+    if (ph == PHASES - 1 && wave < 4u && tiles > 1u) issue_rows(1u, 0u, 2u);
     wg_barrier();
     // this wave's digits of this phase's tokens: sub-blocks 0 .. 15 of its two super-blocks, operand row col (= 4 t + d)
     // and half g of the sub-block; operand rows of tokens the kernel is not built for stay zero
@@ -243,7 +247,10 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
     }
     wg_barrier();                                    // the digits are read: the next phase's, or the tile's rows, may come
   }
-  if (wave >= 4u && tiles > 1u) issue(1u);
+  if (tiles > 1u) {
+    if (wave < 4u) issue_rows(1u, 2u, 4u);
+    else issue(1u);
+  }
 
   // ---- tiles --------------------------------------------------------------------------------------------------------
   // A tile's results leave while the next tile is multiplied: every wave adds up its share of them (4 NTOK of the
@@ -272,8 +279,8 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
   };
   for (u32 tile = 0; tile < tiles; ++tile) {
     // tile `tile` has landed when no more of this wave's operations are outstanding than were issued behind its copies:
-    // the next tile's copies, and the stores of the tiles tile - 3 and tile - 2 (issued in the two rounds before)
-    wait_vm(tile + 1u < tiles ? per_tile + (tile >= 3u ? 2u : tile >= 2u ? 1u : 0u) : 0u);
+    // the next tile's copies, and the store of the tile tile - 2 (issued in the round before, ahead of those copies)
+    wait_vm(tile + 1u < tiles ? per_tile + (tile >= 2u ? 1u : 0u) : 0u);
     wg_barrier();
     // this wave's part of the tile goes to registers, so that the buffer can take the tile after next while this one is
     // multiplied: two tiles on their way at any time
@@ -292,8 +299,9 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
       if (sbi == 0u ? active0 : active1)
         asm volatile("" : "+v"(hdr2[sbi]), "+v"(pc2[sbi][0]), "+v"(pc2[sbi][1]), "+v"(pc2[sbi][2]), "+v"(pc2[sbi][3]));
     wg_barrier();                                    // every wave has its part (and wrote its share of the tile before): the buffer is free
-    if (tile + 2u < tiles) issue(tile + 2u);
+    const bool more = tile + 2u < tiles;             // the tile after next: its copies are issued a row at a time between the MFMAs below
     if (tile > 0u) reduce_store(tile - 1u);
+    if (more && !active0) issue(tile + 2u);          // (a wave without a super-block of its own has no MFMAs to put them between)
     float y[NA];
 #pragma unroll
     for (int aa = 0; aa < NA; ++aa) y[aa] = 0.0f;
@@ -333,6 +341,7 @@ __device__ __forceinline__ void q4k_rows(const float* __restrict__ a, const uint
         const i32x4 bhi = {static_cast<int>((pc[ch].x >> 4) & 0x0F0F0F0Fu), static_cast<int>((pc[ch].y >> 4) & 0x0F0F0F0Fu),
                            static_cast<int>((pc[ch].z >> 4) & 0x0F0F0F0Fu), static_cast<int>((pc[ch].w >> 4) & 0x0F0F0F0Fu)};
         const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if (more && sbi == 0u) issue_rows(tile + 2u, ch, ch + 1u);
         const i32x16 dlo = __builtin_amdgcn_mfma_i32_32x32x32_i8(dig[8 * sbi + 2 * ch], blo, zero, 0, 0, 0);
         const i32x16 dhi = __builtin_amdgcn_mfma_i32_32x32x32_i8(dig[8 * sbi + 2 * ch + 1], bhi, zero, 0, 0, 0);
 #pragma unroll

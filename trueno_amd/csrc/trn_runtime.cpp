@@ -565,7 +565,7 @@ bool gemm_few_tokens_by_engine(const DeviceKernels& d, Fmt f, uint32_t m, uint32
 // The integer matrix-core kernel (kquant_few_i8.hip.h): Q4_K, two to four tokens, a row of W within one slab of 4096
 // columns.  One workgroup per CU at most (its LDS), each with a run of rows that is a multiple of the tile's 32.
 // Times in microseconds measured on MI355X (cold weights, k = 4096; n = 1024, 4096, 11008, 14336, 32000): two tokens
-// 6.2, 6.6, 10.0, 10.6, 18.1; four tokens 8.4, 8.7, 12.5, 13.1, 21.6 - about 2.1 + 0.7 m (m = 2 or 4: what the kernel is
+// 6.0, 6.2, 9.6, 10.3, 17.5; four tokens 8.4, 8.4, 11.7, 12.3, 20.0 - about 2.1 + 0.7 m (m = 2 or 4: what the kernel is
 // built for) to make the digits and for the launch, and 4 per tile of 32 rows that a workgroup takes.  The other ways took, for two and four tokens, 4.9 / 5.1 (the
 // GEMV engine, a pass per token), 7.2 / 9.2, 12.0 / 14.6, 14.8 / 14.8, 23.4 / 23.6 (the f16 matrix-core form).
 constexpr uint32_t kFewRowPad = 32u;
