@@ -3,6 +3,7 @@ from __future__ import annotations
 
 import json
 import os
+import tempfile
 
 import numpy as np
 
@@ -18,7 +19,8 @@ SB = {"q4k": 144, "q5k": 176, "q6k": 210}
 # sampling margin - both errors are sums over a few thousand rounding errors, so their ratio scatters by about
 # 1 / sqrt(rows) around its expectation (1.6 % with 4096 rows, 2.2 % with 2048, 3.1 % with 1024).
 REF_SLACK = 1.05
-RATIO_LOG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "ref_order_ratios.jsonl")
+# where the ratios go: a file named by TRN_RATIO_LOG, else one in the temporary directory
+RATIO_LOG = os.environ.get("TRN_RATIO_LOG") or os.path.join(tempfile.gettempdir(), "trueno_ref_order_ratios.jsonl")
 
 
 def record_ratio(kind: str, fmt: str, m: int, n: int, k: int, rows: int, ours: float, ref: float) -> None:
