@@ -316,6 +316,24 @@ def test_gemm_few_tokens_on_the_integer_cores(gpu, n, k, m):
     assert not np.array_equal(c, other)                      # (two orders of summation: the same bits would mean one path ran twice)
 
 
+@pytest.mark.parametrize("n,k,m", [(20000, 4096, 3), (40000, 4096, 2), (30000, 1024, 4), (70000, 256, 4)])
+def test_gemm_few_tokens_several_tiles_per_workgroup(gpu, n, k, m):
+    """Three to nine tiles per workgroup: the copies of the tile after next are issued between the products of the
+    current one, and a tile's results leave while the next is multiplied (rows of 16, 4 and 1 super-blocks: four, two and
+    one of the eight waves have products of their own)."""
+    buf, a = kq.gen_matrix("q4k", 810 + m, n, k), kq.gen_x(820 + m, m, k)
+    try:
+        _tune("gemm_few", 1)
+        c = gpu_gemm(gpu, "q4k", buf, a, m, n, k)
+    finally:
+        _tune("gemm_few", 0)
+    want = _c64("q4k", buf, a, n, k)
+    assert np.all(np.isfinite(c)) and kq.rel_l2(c, want) <= TOL
+    for i in range(m):                                       # every token, and the ends of the matrix on their own
+        assert kq.rel_l2(c[i], want[i]) <= TOL
+        assert kq.rel_l2(c[i, -40:], want[i, -40:]) <= TOL and kq.rel_l2(c[i, :40], want[i, :40]) <= TOL
+
+
 @pytest.mark.parametrize("m", (2, 4))
 def test_gemm_few_tokens_no_worse_than_reference_order_f32(gpu, coracle, m):
     n, k = 2048, 4096
