@@ -16,7 +16,7 @@ last layer's outputs and the logits are checked against fp64 on their actual inp
 GEMVs wired as the strictly serial chain of a decoder (q,k,v <- h; o <- q; gate,up <- o; down <- gate;
 h <- down) are timed too: `strict_decoder_chain` in `config`.
 
-Prints one JSON line.  `per_pass_us` (in `extra`): minimum, median and maximum of the K timed passes, from one HIP event
+Prints one JSON line.  `per_pass_us` (in `extra`): minimum, median and maximum of the K timed passes (and all K in order), from one HIP event
 between consecutive passes of the timed region itself.  `roofline`: the dominant kernel, kq_gemv_many (the two launches
 of a pass that take their many entries from tables in device memory: the 160 q, k, v, gate, up matrices, then the 64 o and
 down matrices; the head alone runs kq_gemv_group).  Its launches are timed with HIP events on their stream in a second
@@ -53,7 +53,9 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=10, help="untimed passes first (the clocks take some ten milliseconds of load to settle)")
+    ap.add_argument("--warmup", type=int, default=40,
+                    help="untimed passes first (a pass is 0.7 ms and the clocks take some 20 ms of load to settle: with 10 warm-up passes the "
+                         "first 14 timed ones still fell from 850 to 720 us)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the tables of configurations 1, 2, 3 and 5 and of the path's neighbours")
     ap.add_argument("--executors", action="store_true", help="also time the opt-in one-launch executor (batch_mode 1; slower than launches on every list)")
@@ -160,8 +162,9 @@ def main() -> int:
     # ---- timed region: W warm-up passes, then exactly K passes ------------------------------------------------
     ms_per_step, gpu_ms_per_step = run_passes(args.steps, args.warmup, events=pass_events, marks=True)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
-    per_pass = sorted(elapsed_ms(pass_events[i], pass_events[i + 1]) * 1e3 for i in range(args.steps))
-    per_pass_us = {"min": round(per_pass[0], 1), "median": round(per_pass[len(per_pass) // 2], 1), "max": round(per_pass[-1], 1)}
+    in_order = [round(elapsed_ms(pass_events[i], pass_events[i + 1]) * 1e3, 1) for i in range(args.steps)]
+    per_pass = sorted(in_order)
+    per_pass_us = {"min": per_pass[0], "median": per_pass[len(per_pass) // 2], "max": per_pass[-1], "in_order": in_order}
 
     # ---- what the timed passes left behind, against fp64 on the actual inputs: the last layer and the logits ------
     def norm64(v, eps=1e-6):
