@@ -198,8 +198,10 @@ TRN_API trn_status trn_q4k_gemm_fused(trn_stream stream, trn_dptr a, trn_dptr b_
  * overtake.  Up to sixteen entries travel in the kernel's arguments; a launch of more takes them from tables in
  * device memory, which are made when a list is first seen on a stream and kept for as long as the same list (the
  * same descriptors, byte for byte) comes again - up to eight lists per stream, the one used longest ago makes room.
- * While the stream is being captured into a graph launches hold at most sixteen entries (nothing is copied or
- * allocated).  What an entry computes does not depend on the company it is launched in: the results are, bit for
+ * While the stream is being captured into a graph nothing is copied or allocated: a list that the same stream has
+ * issued eagerly before (and whose tables it still holds) is recorded with those launches, and the tables a graph
+ * reads are then kept until the process ends (a few hundred KB per captured list); any other list is recorded as
+ * launches of at most sixteen entries.  What an entry computes does not depend on the company it is launched in: the results are, bit for
  * bit, those of one launch per entry in list order.
  * With trn_set_tuning("batch_mode", 1), and when every entry meets the fast kernels' alignment (x 16 B,
  * W 16 B / 2 B for Q6_K), the list runs as ONE cooperative launch of resident workgroups: the list is cut in

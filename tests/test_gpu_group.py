@@ -301,3 +301,64 @@ def test_a_list_captured_into_a_hip_graph_replays_to_the_same_bits(gpu):
     finally:
         hip.hipGraphExecDestroy(gexec)
         hip.hipGraphDestroy(graph)
+
+
+def test_a_capture_of_a_list_issued_before_takes_its_large_launch(gpu):
+    """A list of more than sixteen independent entries that the stream has issued eagerly is captured as the ONE launch it
+    is (its tables exist already: nothing is allocated under capture); the replays give the eager bits, also after the
+    plan has been pushed out of the stream's cache by nine other lists - the tables a graph may read are kept."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphGetNodes.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_size_t)]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    ctx, stream = gpu
+
+    def make(seed, entries):
+        x = t.GpuBuffer.from_host(ctx, kq.gen_x(seed, 4096))
+        outs, keep, batch = [], [x], t.GemvBatch()
+        for i in range(entries):
+            fmt, n, k = ("q4k", "q6k", "q5k")[i % 3], 100 + 61 * i, 256 * (1 + i % 16)
+            w = t.GpuBuffer.from_host(ctx, kq.gen_matrix(fmt, seed * 100 + i, n, k))
+            y = t.GpuBuffer.from_host(ctx, np.full(n, np.nan, np.float32))
+            keep.append(w)
+            outs.append(y)
+            batch.add(fmt, k, n, y, w, x, i % 2)
+        return batch, outs, keep
+
+    batch, outs, keep = make(5, 24)
+    assert max(batch.plan()) == 0                      # one launch
+    batch.launch(stream)                               # eager: makes the plan and its tables
+    stream.synchronize()
+    want = [y.copy_to_host() for y in outs]
+    assert all(np.all(np.isfinite(w)) for w in want)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.raw(), 0) == 0
+    batch.launch(stream)
+    assert hip.hipStreamEndCapture(stream.raw(), C.byref(graph)) == 0
+    nodes = C.c_size_t(0)
+    assert hip.hipGraphGetNodes(graph, None, C.byref(nodes)) == 0 and nodes.value == 1, nodes.value
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    others = []
+    try:
+        for rep in range(4):
+            for y, w in zip(outs, want):
+                y.copy_from_host(np.full(len(w), np.nan, np.float32))
+            assert hip.hipGraphLaunch(gexec, stream.raw()) == 0
+            stream.synchronize()
+            for i, (y, w) in enumerate(zip(outs, want)):
+                assert np.array_equal(y.copy_to_host().view(np.uint32), w.view(np.uint32)), (rep, i)
+            if rep == 1:                               # nine other lists: the captured list's plan leaves the cache
+                for s in range(9):
+                    others.append(make(20 + s, 18 + s))
+                    others[-1][0].launch(stream)
+                stream.synchronize()
+            batch.launch(stream)                       # eager work between the replays (after rep 1: a new plan, new tables)
+            stream.synchronize()
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)

@@ -1661,6 +1661,7 @@ struct ListPlan {
   std::vector<trn_gemv_desc> key;
   int epoch = -1;
   uint64_t used = 0;           // when it was used last (g_plan_clock)
+  bool in_a_graph = false;     // a stream capture has recorded launches that read this plan's device tables
   std::vector<PlannedLaunch> launches;
 };
 // A few plans per stream (a decoder may issue the layers' lists one by one, or alternate between lists): the one used
@@ -1669,12 +1670,17 @@ constexpr size_t kPlansPerStream = 8;
 uint64_t g_plan_clock = 0;
 std::map<std::tuple<int, hipStream_t, bool>, std::vector<ListPlan>> g_list_plans;     // by device, stream and "may make large launches"; under g_ws_mutex
 
+// Tables that a captured graph may still read are never freed (a graph can be replayed for as long as the process
+// lives, on any stream): they are a few hundred KB per list, and there are as many as lists were captured.
+size_t g_table_bytes_left_to_graphs = 0;
 void free_plan_tables(ListPlan* plan) {
   for (PlannedLaunch& l : plan->launches)
     if (l.many.dev) {
-      (void)hipFree(l.many.dev);
+      if (plan->in_a_graph) g_table_bytes_left_to_graphs += l.many.host.size() * 4u;
+      else (void)hipFree(l.many.dev);
       l.many.dev = nullptr;
     }
+  plan->in_a_graph = false;
 }
 void release_list_plans(hipStream_t stream) {       // under g_ws_mutex; the stream is idle
   for (auto it = g_list_plans.begin(); it != g_list_plans.end();) {
@@ -1779,12 +1785,26 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
     (void)hipGetLastError();
     capturing = hipStreamCaptureStatusNone;
   }
-  const bool many_ok = capturing == hipStreamCaptureStatusNone;
+  bool many_ok = capturing == hipStreamCaptureStatusNone;
   std::lock_guard<std::mutex> lock(g_ws_mutex);
-  std::vector<ListPlan>& plans = g_list_plans[std::make_tuple(dev, stream, many_ok)];      // (a capture has plans of its own)
-  ListPlan* found = nullptr;
-  for (ListPlan& p : plans)
-    if (p.epoch == g_tune_epoch && p.key.size() == count && std::memcmp(p.key.data(), descs, size_t(count) * sizeof(trn_gemv_desc)) == 0) found = &p;
+  auto find_in = [&](std::vector<ListPlan>& list) -> ListPlan* {
+    for (ListPlan& p : list)
+      if (p.epoch == g_tune_epoch && p.key.size() == count && std::memcmp(p.key.data(), descs, size_t(count) * sizeof(trn_gemv_desc)) == 0) return &p;
+    return nullptr;
+  };
+  // A capture of a list that this stream has already issued eagerly takes that plan, tables and all: nothing is built,
+  // copied or allocated, and the tables are then kept for as long as the process lives (free_plan_tables).
+  if (!many_ok) {
+    auto eager = g_list_plans.find(std::make_tuple(dev, stream, true));
+    if (eager != g_list_plans.end()) {
+      if (ListPlan* p = find_in(eager->second)) {
+        p->in_a_graph = true;
+        many_ok = true;
+      }
+    }
+  }
+  std::vector<ListPlan>& plans = g_list_plans[std::make_tuple(dev, stream, many_ok)];      // (a capture of anything else has plans of its own)
+  ListPlan* found = find_in(plans);
   const bool same = found != nullptr;
   if (!same) {
     if (plans.size() < kPlansPerStream) {
