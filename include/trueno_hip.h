@@ -322,7 +322,8 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * "gemv_stream_off": 1 = no matrix streams its rows through LDS (every GEMV loads its rows into registers straight from
  * memory; same bits); "gemv_stream_q6k": 1 = Q6_K matrices of up to 4096 columns stream too (slower, measured);
  * "gemv_stream_waves": waves per workgroup of a single streamed GEMV (0 = 4); "gemv_stream_min_rows": a single GEMV
- * streams when a wave gets at least this many rows (0 = 16); "gemv_stream_cost": percent of its bytes a streamed entry
+ * streams when a wave gets at least this many rows (0 = 16); "group_stream_min_rows": the same for an entry of a launch
+ * of up to sixteen entries (0 = 16); "gemv_stream_cost": percent of its bytes a streamed entry
  * counts for when a launch shares out its workgroups (0 = 95).
  * "gemm_few": the Q4_K product of two to four tokens on the integer matrix cores - 0 = where its estimated time is the
  * lowest, 1 = wherever it can run, 2 = never.

@@ -117,6 +117,7 @@ std::atomic<int> g_tune_stream_q6k{0};      // 1: Q6_K one-slab GEMVs stream thr
 std::atomic<int> g_tune_stream_cost{0};     // percent of its bytes a streamed entry counts for when a grouped launch shares out its workgroups (0: default)
 std::atomic<int> g_tune_stream_min_rows{0}; // a single GEMV streams when a wave gets at least this many rows (0: default)
 std::atomic<int> g_tune_many_waves{0};      // waves per workgroup of a launch of more than sixteen entries (0: 12)
+std::atomic<int> g_tune_group_stream_min_rows{0};  // an entry of a launch of up to sixteen streams when a wave gets at least this many rows (0: default)
 std::atomic<int> g_tune_many_item_kb{0};    // what a further piece of work costs a workgroup of such a launch, in KB of weights (0: default)
 std::atomic<int> g_tune_many_slab_weight{0};  // percent such a launch adds to an entry's bytes per slab of 4096 columns beyond the first (0: default)
 std::atomic<int> g_tune_stream_waves{0};    // waves per workgroup of a single streamed GEMV (0: default)
@@ -755,6 +756,9 @@ constexpr uint32_t kGroupMax = 16;     // entries one grouped launch can hold (k
 constexpr double kSlabCost = 0.4;
 // what a streamed entry's bytes cost against an entry's on the register path (launch_gemv_group)
 constexpr double kStreamCost = 0.95;
+// rows a wave must get for an entry of a launch of up to sixteen to stream: the strict decoder chain 1370 / 1381 / 1356 / 1338 / 1336 /
+// 1334 us with 1 / 4 / 8 / 12 / 16 / 24 (its launches of one to three entries leave a wave 6-11 rows); the pass with shared buffers within its scatter
+constexpr double kGroupStreamMinRows = 16.0;
 // launches of more than sixteen entries (plan_gemv_many): weight per further slab and what a piece of work costs a workgroup
 // (KB of weights).  The 7B pass: 730 / 718 / 704 / 702 / 702 / 708 / 711 us with 40 / 30 / 25 / 20 / 15 / 10 / 5 % per slab (with 40 %
 // the workgroups with the one-slab o matrices ended 35 us after those with the three-slab down matrices); the cost of a piece
@@ -1442,30 +1446,39 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   // the wide entry's workgroups end 5 us after the others; counting its bytes 1.6-1.8 times is best (0.4 per
   // further slab of 4096 columns; "group_slab_weight" overrides the percentage.  The 7B pass in launches of sixteen
   // entries: 932 / 875 / 832 / 800 / 794 / 803 / 880 us with 1 / 10 / 20 / 30 / 40 / 50 / 70 percent).
-  auto cost_of = [&](const trn_gemv_desc& e) {
-    const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
-    const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
-    // a streamed entry's bytes arrive faster than those of an entry on the register path
-    const bool streamed = stream_ok(e.fmt, e.k, e.n) &&
-                          uint64_t(e.k) * 4u + kLdsScratch + waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) + kGemvRowsPerBatch * 4u <= kStreamLdsLimit;
-    const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
-    return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u)) * (streamed ? stream_cost : 1.0);
-  };
-  for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of(descs[i]);
   // the kernels hold 3 waves per SIMD, 12 per CU
   const uint32_t per_cu = g_tune_blocks_per_cu > 0 ? uint32_t(g_tune_blocks_per_cu) : std::max(1u, 12u / waves);
   const double target = double(d->cu_count) * per_cu;
+  auto plain_cost_of = [&](const trn_gemv_desc& e) {
+    const uint32_t slabs = std::min((e.k / 256u + 15u) / 16u, waves);
+    const double per_slab = g_tune_slab_weight > 0 ? int(g_tune_slab_weight) / 100.0 : kSlabCost;
+    return double(e.n) * (e.k / 256u) * kSbBytes[e.fmt - 4] * (1.0 + per_slab * (slabs - 1u));
+  };
+  double plain_total = 0.0;
+  for (uint32_t i = 0; i < len; ++i) plain_total += plain_cost_of(descs[i]);
+  // An entry of one slab streams its rows through LDS when the rings of all waves fit beside its vector and a wave gets
+  // enough rows to make the ring pay (by the entry's share of the workgroups: a ring is filled two batches ahead and
+  // its start costs what a few rows cost).
+  const double min_rows = g_tune_group_stream_min_rows > 0 ? double(int(g_tune_group_stream_min_rows)) : kGroupStreamMinRows;
+  bool streams[kGroupMax] = {};
+  for (uint32_t i = 0; i < len; ++i) {
+    const trn_gemv_desc& e = descs[i];
+    const double share = std::max(1.0, target * plain_cost_of(e) / std::max(plain_total, 1.0));
+    streams[i] = stream_ok(e.fmt, e.k, e.n) && double(e.n) / share / waves >= min_rows &&
+                 uint64_t(e.k) * 4u + kLdsScratch + waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]) + kGemvRowsPerBatch * 4u <= kStreamLdsLimit;
+  }
+  auto cost_of_i = [&](uint32_t i) {
+    // a streamed entry's bytes arrive faster than those of an entry on the register path
+    const double stream_cost = g_tune_stream_cost > 0 ? int(g_tune_stream_cost) / 100.0 : kStreamCost;
+    return plain_cost_of(descs[i]) * (streams[i] ? stream_cost : 1.0);
+  };
+  for (uint32_t i = 0; i < len; ++i) total_bytes += cost_of_i(i);
   GemvGroupHost g{};
   uint32_t first[kGroupMax + 1] = {};
   uint32_t lds = 0;
   // rows per workgroup and workgroups of entry i when it is given `share` workgroups (0 rows: it does not fit the engine)
   // an entry of one slab streams its rows through LDS when the rings of all waves fit beside its vector
-  auto ring_of = [&](uint32_t i) -> uint32_t {
-    const trn_gemv_desc& e = descs[i];
-    if (!stream_ok(e.fmt, e.k, e.n)) return 0u;
-    const uint32_t ring = waves * 2u * stream_slot_bytes(kSbBytes[e.fmt - 4]);
-    return uint64_t(e.k) * 4u + kLdsScratch + ring + kGemvRowsPerBatch * 4u <= kStreamLdsLimit ? ring : 0u;
-  };
+  auto ring_of = [&](uint32_t i) -> uint32_t { return streams[i] ? waves * 2u * stream_slot_bytes(kSbBytes[descs[i].fmt - 4]) : 0u; };
   struct Cut { uint64_t rows; uint32_t grid; };
   auto cut_of = [&](uint32_t i, uint64_t share) {
     const trn_gemv_desc& e = descs[i];
@@ -1487,7 +1500,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
   Cut cut[kGroupMax] = {};
   uint64_t total_grid = 0;
   for (uint32_t i = 0; i < len; ++i) {
-    share[i] = std::max<uint64_t>(1, uint64_t(target * cost_of(descs[i]) / total_bytes + 0.5));
+    share[i] = std::max<uint64_t>(1, uint64_t(target * cost_of_i(i) / total_bytes + 0.5));
     cut[i] = cut_of(i, share[i]);
     if (cut[i].rows == 0) return hipErrorInvalidValue;
     total_grid += cut[i].grid;
@@ -1513,7 +1526,7 @@ hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gem
     Cut best_cut{};
     uint64_t best_share = 0;
     for (uint32_t i = 0; i < len; ++i) {
-      const double per_wg = cost_of(descs[i]) / double(descs[i].n) * double(cut[i].rows);
+      const double per_wg = cost_of_i(i) / double(descs[i].n) * double(cut[i].rows);
       if (per_wg <= most) continue;
       uint64_t sh = share[i];
       Cut c = cut[i];
@@ -2011,6 +2024,7 @@ trn_status trn_set_tuning(const char* key, int value) {
   if (!std::strcmp(key, "gemv_stream_off")) { g_tune_stream_off = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_waves")) { g_tune_stream_waves = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "many_waves")) { g_tune_many_waves = value; return TRN_SUCCESS; }
+  if (!std::strcmp(key, "group_stream_min_rows")) { g_tune_group_stream_min_rows = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "many_item_kb")) { g_tune_many_item_kb = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "many_slab_weight")) { g_tune_many_slab_weight = value; return TRN_SUCCESS; }
   if (!std::strcmp(key, "gemv_stream_q6k")) { g_tune_stream_q6k = value; return TRN_SUCCESS; }
