@@ -588,6 +588,12 @@ hipError_t launch_gemm_few(DeviceKernels* d, hipStream_t stream, uint64_t a, uin
   return hipModuleLaunchKernel(d->gemm_few[idx], grid, 1, 1, 512, 1, 1, lds, stream, args, nullptr);
 }
 
+constexpr double kBigAloneBytes = 64e6;      // from this size on a matrix alone takes the list kernel (launch_gemm_like, trn_kquant_gemv_batch)
+bool list_groupable(DeviceKernels* dk, const trn_gemv_desc& d);
+extern "C" {      // (defined further down inside the extern "C" part of the file: the same language linkage here)
+hipError_t launch_gemv_group(DeviceKernels* d, hipStream_t stream, const trn_gemv_desc* descs, uint32_t len);
+}
+
 // Which kernel takes a product of m >= 1 tokens: the integer matrix cores (Q4_K, two to four tokens, where their fitted
 // time is below the other ways'), the f16 matrix cores, or the GEMV engine with a pass per token (also: whatever the
 // matrix-core forms cannot take).  A forced cut of the f16 form (tuning) takes that form.
@@ -623,6 +629,13 @@ hipError_t launch_gemm_like(Fmt f, hipStream_t stream, uint64_t a, uint64_t w, u
   void* gemv_args[] = {&c, &w, &a, &k, &n, &flags};   // the by-name kernel takes the first five
   void* gemm_args[] = {&a, &w, &c, &m, &n, &k};
   void** args = is_gemv ? gemv_args : gemm_args;
+  // A large matrix alone is 2-5 us faster as a launch of the list kernel with one entry (workgroups of 8 waves that hand
+  // their rows out among themselves) than through the single kernel: Q6_K 32000 x 4096, 108 MB, 22.7 against 27.2 us.
+  if (is_gemv && flags == 0 && !g_tune_group_off && double(n) * (k / 256u) * kSbBytes[f] >= kBigAloneBytes) {
+    trn_gemv_desc one{};
+    one.fmt = uint32_t(f) + 4u; one.k = k; one.n = n; one.y = c; one.w = w; one.x = a;
+    if (list_groupable(d, one)) return launch_gemv_group(d, stream, &one, 1);
+  }
   GemvGeometry g;
   if (is_gemv && gemv_fast_ok(f, c, w, a) && stream_ok(uint32_t(f) + 4u, k, n)) {
     g = stream_geometry(*d, f, k, n);
@@ -1869,7 +1882,7 @@ trn_status trn_kquant_gemv_batch(trn_stream s, const trn_gemv_desc* descs, uint3
     const trn_gemv_desc& head = descs[members[0]];
     // a large matrix alone (the 108 MB head of the 7B pass) is 2-4 us faster as a group of one: workgroups of 8 waves that
     // hand their rows out among themselves; smaller ones alone (37 MB, 9 MB) are slower that way
-    const bool big_single = list_groupable(dk, head) && double(head.n) * (head.k / 256u) * kSbBytes[head.fmt - 4] >= 64e6;
+    const bool big_single = list_groupable(dk, head) && double(head.n) * (head.k / 256u) * kSbBytes[head.fmt - 4] >= kBigAloneBytes;
     if (pl.many.dev) {
       uint64_t wgs = reinterpret_cast<uint64_t>(pl.many.dev), items = wgs + pl.many.off_items, hot = wgs + pl.many.off_hot,
                cold = wgs + pl.many.off_cold;
