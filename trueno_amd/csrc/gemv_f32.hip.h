@@ -36,7 +36,7 @@ __device__ __forceinline__ void fast_body(float* __restrict__ y, const float* __
     float xv[kUnroll];
 #pragma unroll
     for (u32 u = 0; u < kUnroll; ++u) {
-      v[u] = ap[static_cast<size_t>(k + u * kWaves) * stride4];
+      v[u] = __builtin_nontemporal_load(ap + static_cast<size_t>(k + u * kWaves) * stride4);   // (the matrix is read once, in whole lines)
       xv[u] = x[k + u * kWaves];
     }
 #pragma unroll
@@ -46,7 +46,7 @@ __device__ __forceinline__ void fast_body(float* __restrict__ y, const float* __
     }
   }
   for (; k < k1; k += kWaves) {
-    const f32x4 v = ap[static_cast<size_t>(k) * stride4];
+    const f32x4 v = __builtin_nontemporal_load(ap + static_cast<size_t>(k) * stride4);
     const float xk = x[k];
     acc.x = fmaf(v.x, xk, acc.x); acc.y = fmaf(v.y, xk, acc.y); acc.z = fmaf(v.z, xk, acc.z); acc.w = fmaf(v.w, xk, acc.w);
   }
