@@ -262,7 +262,7 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       if (lane == 0) asm volatile("ds_write_b32 %0, %1" ::"v"(lds_ss + 4u * g), "v"(sg) : "memory");
     }
     if (e.gamma) {
-      const f32x4 gm = reinterpret_cast<const f32x4*>(e.gamma)[64u * g + lane];
+      const f32x4 gm = KQ_GLOBAL(f32x4, e.gamma)[64u * g + lane];
       v = f32x4{__fmul_rn(v.x, gm.x), __fmul_rn(v.y, gm.y), __fmul_rn(v.z, gm.z), __fmul_rn(v.w, gm.w)};
     }
     asm volatile("ds_write_b128 %0, %1" ::"v"(lds_x + 16u * Q::swz(64u * g + lane)), "v"(v) : "memory");
@@ -281,9 +281,9 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
     }
   }
   for (u32 g = wave + kXPre * waves; g < xgroups; g += waves) {     // (workgroups of fewer than four waves)
-    f32x4 v = reinterpret_cast<const f32x4*>(e.x)[64u * g + lane];
+    f32x4 v = KQ_GLOBAL(f32x4, e.x)[64u * g + lane];
     if (swiglu) {
-      const f32x4 g2 = reinterpret_cast<const f32x4*>(e.x2)[64u * g + lane];
+      const f32x4 g2 = KQ_GLOBAL(f32x4, e.x2)[64u * g + lane];
       v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
     }
     stage(g, v);
@@ -362,8 +362,8 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
     const u32 row = row0 + t;
     if (row < n_dim) {
       float r = part[t] * scale;
-      if (e.residual) r = __fadd_rn(r, e.residual[row]);
-      e.y[row] = r;
+      if (e.residual) r = __fadd_rn(r, KQ_GLOBAL(float, e.residual)[row]);
+      KQ_GLOBAL_MUT(float, e.y)[row] = r;
     }
   }
   return true;
@@ -384,7 +384,8 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
   if (block_threads < 64u || (block_threads & 63u) != 0u) return true;
   if constexpr (!COHERENT)      // (the resident executor keeps the register path: its launcher never sets the flag)
     if ((e.flags & CHAIN_STREAM_LDS) && wait_counter == nullptr) return chain_step_stream<FMT, U>(e, lds4, row0, rows_per_block, block_threads);
-  const u32 tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = block_threads >> 6;
+  const u32 tid = threadIdx.x, lane = tid & 63u, waves = block_threads >> 6;
+  const u32 wave = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(tid >> 6)));   // (the same in every lane: scalar)
   const u32 k_dim = e.k, n_dim = e.n, nsb = k_dim >> 8;
   const u32 slabs = (nsb + 15u) >> 4;
   const u32 sw_count = slabs < waves ? slabs : waves;
@@ -399,12 +400,11 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
   auto issue = [&](u32 slab, u32 b) {
     const u32 sb = slab * 16u + sbl;
     const u32 sbc = sb < nsb ? sb : nsb - 1;
-    const uint8_t* col = e.w + static_cast<size_t>(sbc) * Q::SB;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       u32 row = row0 + b * U + u;
       row = row < n_dim ? row : n_dim - 1;
-      Q::load(regs[u], col + row * row_bytes, c);
+      Q::load(regs[u], e.w + row * row_bytes, sbc * Q::SB, c);     // (a row is tens of KB at most: its vector must fit in LDS)
     }
   };
   // Activations.  Alone on the stream (no barrier to wait for) they are requested BEFORE the weights: loads
@@ -427,11 +427,11 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
   auto load_x = [&](u32 u) {
     f32x4 v;
     if constexpr (COHERENT) v = coherent16(x_rsrc, u);
-    else v = x4[u];
+    else v = KQ_GLOBAL(f32x4, x4)[u];
     if (e.flags & CHAIN_SWIGLU_INPUT) {
       f32x4 g2;
       if constexpr (COHERENT) g2 = coherent16(x2_rsrc, u);
-      else g2 = reinterpret_cast<const f32x4*>(e.x2)[u];
+      else g2 = KQ_GLOBAL(f32x4, e.x2)[u];
       v = f32x4{swiglu1(v.x, g2.x), swiglu1(v.y, g2.y), swiglu1(v.z, g2.z), swiglu1(v.w, g2.w)};
     }
     return v;
@@ -467,7 +467,7 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
       if (lane == 0) group_ss[g] = sg;
     }
     if (e.gamma) {                      // weights of the normalisation, never written inside a launch
-      const f32x4 gm = reinterpret_cast<const f32x4*>(e.gamma)[64u * g + lane];
+      const f32x4 gm = KQ_GLOBAL(f32x4, e.gamma)[64u * g + lane];
       v = f32x4{__fmul_rn(v.x, gm.x), __fmul_rn(v.y, gm.y), __fmul_rn(v.z, gm.z), __fmul_rn(v.w, gm.w)};
     }
     lds4[Q::swz(64u * g + lane)] = v;
@@ -543,12 +543,12 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
       float r = s * scale;
       if constexpr (COHERENT) {
         if (e.residual)
-          r = __fadd_rn(r, __uint_as_float(__hip_atomic_load(reinterpret_cast<const u32*>(e.residual) + row, __ATOMIC_RELAXED,
+          r = __fadd_rn(r, __uint_as_float(__hip_atomic_load(KQ_GLOBAL(u32, e.residual) + row, __ATOMIC_RELAXED,
                                                              __HIP_MEMORY_SCOPE_AGENT)));
-        __hip_atomic_store(reinterpret_cast<u32*>(e.y) + row, __float_as_uint(r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(KQ_GLOBAL_MUT(u32, e.y) + row, __float_as_uint(r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
-        if (e.residual) r = __fadd_rn(r, e.residual[row]);
-        e.y[row] = r;
+        if (e.residual) r = __fadd_rn(r, KQ_GLOBAL(float, e.residual)[row]);
+        KQ_GLOBAL_MUT(float, e.y)[row] = r;
       }
     }
   }

@@ -32,13 +32,20 @@ struct __attribute__((packed, aligned(2))) ld64_a2 { u32x2 v; };
 struct __attribute__((packed, aligned(1))) ld32_a1 { u32 v; };
 struct __attribute__((packed, aligned(2))) ld16_a2 { uint16_t v; };
 
-__device__ __forceinline__ u32x4 load128_a2(const uint8_t* p) { return reinterpret_cast<const ld128_a2*>(p)->v; }
-__device__ __forceinline__ u32x2 load64_a2(const uint8_t* p) { return reinterpret_cast<const ld64_a2*>(p)->v; }
-__device__ __forceinline__ u32 load32_a1(const uint8_t* p) { return reinterpret_cast<const ld32_a1*>(p)->v; }
-__device__ __forceinline__ u32 load16_a2(const uint8_t* p) { return reinterpret_cast<const ld16_a2*>(p)->v; }
-__device__ __forceinline__ u32x4 load128(const uint8_t* p) { return *reinterpret_cast<const u32x4*>(p); }
-__device__ __forceinline__ u32x2 load64(const uint8_t* p) { return *reinterpret_cast<const u32x2*>(p); }
-__device__ __forceinline__ u32 load32(const uint8_t* p) { return *reinterpret_cast<const u32*>(p); }
+// Every pointer these take is a weight matrix in device memory; saying so (address space 1) makes them global_load
+// instructions also where the pointer came out of a table in memory and the compiler could not tell.  A generic pointer
+// is a flat_load, which counts as an LDS access as well: nothing behind it can be waited for on its own, so a wave
+// would wait for both of its rows before it computes the first, and for its rows before it stages the vector.  The
+// engines say the same of the vectors they read and write (KQ_GLOBAL, KQ_GLOBAL_MUT).
+#define KQ_GLOBAL(T, p) (reinterpret_cast<const __attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)))
+#define KQ_GLOBAL_MUT(T, p) (reinterpret_cast<__attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)))
+__device__ __forceinline__ u32x4 load128_a2(const uint8_t* p) { return KQ_GLOBAL(ld128_a2, p)->v; }
+__device__ __forceinline__ u32x2 load64_a2(const uint8_t* p) { return KQ_GLOBAL(ld64_a2, p)->v; }
+__device__ __forceinline__ u32 load32_a1(const uint8_t* p) { return KQ_GLOBAL(ld32_a1, p)->v; }
+__device__ __forceinline__ u32 load16_a2(const uint8_t* p) { return KQ_GLOBAL(ld16_a2, p)->v; }
+__device__ __forceinline__ u32x4 load128(const uint8_t* p) { return *KQ_GLOBAL(u32x4, p); }
+__device__ __forceinline__ u32x2 load64(const uint8_t* p) { return *KQ_GLOBAL(u32x2, p); }
+__device__ __forceinline__ u32 load32(const uint8_t* p) { return *KQ_GLOBAL(u32, p); }
 
 // f16 bits -> f32, exact, subnormals kept (the reference converts with cvt.f32.f16, no .ftz:
 // trueno-gpu/src/ptx/builder.rs:1241-1250).

@@ -417,7 +417,7 @@ __device__ __forceinline__ void dequant_fast_body(float* __restrict__ out, const
     const uint64_t sb = gid >> 2;
     const u32 c = static_cast<u32>(gid & 3u);
     typename Q::Regs r;
-    Q::load(r, w + sb * Q::SB, c);
+    Q::load(r, w + sb * Q::SB, 0u, c);
     float wv[64];
     Q::dequant(r, c, wv);
     float* o = out + sb * 256;

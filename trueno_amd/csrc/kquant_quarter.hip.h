@@ -45,10 +45,13 @@ template <> struct Quarter<FMT_Q4K> {
   static __device__ __forceinline__ u32 value_index(u32 c, u32 j) { return 64u * c + j; }
   static __device__ __forceinline__ u32 sum_index(u32 j) { return j >> 5; }
 
-  static __device__ __forceinline__ void load(Regs& r, const uint8_t* sbp, u32 c) {
-    r.hdr = load128(sbp);
-    r.q0 = load128(sbp + 16 + 32 * c);
-    r.q1 = load128(sbp + 32 + 32 * c);
+  // The block lies `off` bytes behind `base`.  Callers hand in a base that is the same for the whole wave (a row of
+  // the matrix) and keep what differs from lane to lane in the 32-bit offset: the address of a load is then a scalar
+  // register pair plus one vector register, not a 64-bit sum per lane and piece.
+  static __device__ __forceinline__ void load(Regs& r, const uint8_t* base, u32 off, u32 c) {
+    r.hdr = load128(base + off);
+    r.q0 = load128(base + (off + 32u * c) + 16);
+    r.q1 = load128(base + (off + 32u * c) + 32);
   }
 
   // the same three pieces from a copy of the block in LDS (at byte address `blk`)
@@ -143,12 +146,12 @@ template <> struct Quarter<FMT_Q5K> {
   static __device__ __forceinline__ u32 value_index(u32 c, u32 j) { return 64u * c + j; }
   static __device__ __forceinline__ u32 sum_index(u32 j) { return j >> 5; }
 
-  static __device__ __forceinline__ void load(Regs& r, const uint8_t* sbp, u32 c) {
-    r.dd = load32(sbp);
-    r.f24 = load32_a1(sbp + 4 + 3 * c);  // c == 3 also reads qs[0]; masked off below
-    r.q0 = load128(sbp + 16 + 32 * c);
-    r.q1 = load128(sbp + 32 + 32 * c);
-    r.qh = load64(sbp + 144 + 8 * c);
+  static __device__ __forceinline__ void load(Regs& r, const uint8_t* base, u32 off, u32 c) {
+    r.dd = load32(base + off);
+    r.f24 = load32_a1(base + (off + 3u * c) + 4);  // c == 3 also reads qs[0]; masked off below
+    r.q0 = load128(base + (off + 32u * c) + 16);
+    r.q1 = load128(base + (off + 32u * c) + 32);
+    r.qh = load64(base + (off + 8u * c) + 144);
   }
 
   static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {
@@ -248,13 +251,13 @@ template <> struct Quarter<FMT_Q6K> {
   }
   static __device__ __forceinline__ u32 sum_index(u32 j) { return j >> 4; }
 
-  static __device__ __forceinline__ void load(Regs& r, const uint8_t* sbp, u32 c) {
+  static __device__ __forceinline__ void load(Regs& r, const uint8_t* base, u32 off, u32 c) {
     const u32 h = c >> 1, is = c & 1u;
-    r.a = load128_a2(sbp + 64 * h + 16 * is);
-    r.b = load128_a2(sbp + 64 * h + 32 + 16 * is);
-    r.c = load128_a2(sbp + 128 + 32 * h + 16 * is);
-    r.sc = load64_a2(sbp + 192 + 8 * h);
-    r.d = load16_a2(sbp + 208);
+    r.a = load128_a2(base + (off + 64u * h + 16u * is));
+    r.b = load128_a2(base + (off + 64u * h + 16u * is) + 32);
+    r.c = load128_a2(base + (off + 32u * h + 16u * is) + 128);
+    r.sc = load64_a2(base + (off + 8u * h) + 192);
+    r.d = load16_a2(base + off + 208);
   }
 
   static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {       // blocks lie at 2-byte alignment in LDS too
