@@ -391,20 +391,25 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
   const u32 sw_count = slabs < waves ? slabs : waves;
   const u32 groups = waves / sw_count;
   const bool has_rows = row0 < n_dim && nsb != 0;
-  const u32 batches = has_rows ? rows_per_block / U : 0u;
+  // Rows go through two sets of registers, one row each: while a row is computed the wave's next row is on its way into
+  // the other set.  (Two rows per set and no second set - the same registers - leaves the wave idle while it waits:
+  // with three waves to a SIMD the others do not fill that time.  Two sets of two rows do not fit the registers, and a
+  // spilled register that is read back inside the loop waits for every load issued before it, the next rows' included.)
+  constexpr int UR = 1;
+  const u32 batches = has_rows ? rows_per_block / UR : 0u;
   const u32 sw = wave % sw_count, grp = wave / sw_count;
   const bool wave_active = grp < groups && grp < batches;
   const u32 sbl = lane >> 2, c = lane & 3u;
   const size_t row_bytes = static_cast<size_t>(nsb) * Q::SB;
-  typename Q::Regs regs[U];
-  auto issue = [&](u32 slab, u32 b) {
+  typename Q::Regs regs[UR], regs_b[UR];
+  auto issue = [&](typename Q::Regs (&into)[UR], u32 slab, u32 b) {
     const u32 sb = slab * 16u + sbl;
     const u32 sbc = sb < nsb ? sb : nsb - 1;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      u32 row = row0 + b * U + u;
+    for (int u = 0; u < UR; ++u) {
+      u32 row = row0 + b * UR + u;
       row = row < n_dim ? row : n_dim - 1;
-      Q::load(regs[u], e.w + row * row_bytes, sbc * Q::SB, c);     // (a row is tens of KB at most: its vector must fit in LDS)
+      Q::load(into[u], e.w + row * row_bytes, sbc * Q::SB, c);     // (a row is tens of KB at most: its vector must fit in LDS)
     }
   };
   // Activations.  Alone on the stream (no barrier to wait for) they are requested BEFORE the weights: loads
@@ -452,10 +457,10 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
   // The wave that polls a barrier asks for its rows only when the barrier has opened: loads return in order, and the
   // answer to a poll behind weight loads comes late, for the whole workgroup.
   const bool polls = wait_counter != nullptr && wave == 0u;
-  if (!polls) issue(sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
+  if (!polls) issue(regs, sw, wave_active ? grp : 0u);        // the host never launches this engine with k = 0 or n = 0
 
   if (wait_counter && !chain_wait(wait_counter, spin_limit, status, s_flag)) return false;
-  if (polls) issue(sw, wave_active ? grp : 0u);
+  if (polls) issue(regs, sw, wave_active ? grp : 0u);
   if (!has_rows) return true;
 
   float* part = reinterpret_cast<float*>(lds4 + units);
@@ -514,23 +519,37 @@ __device__ __forceinline__ bool chain_step_rows(const ChainEntry& e, u32* wait_c
         sx[Q::sum_index(4 * q)] += (v.x + v.y) + (v.z + v.w);
       }
       const bool handed_out = slabs <= waves && waves >= 8u;   // every wave owns one slab; small workgroups gain nothing
-      for (u32 b = grp; b < batches;) {
-        if (slab != sw || b != grp) issue(slab, b);
-        u32 nb = 0u;                                // the batch after this one, asked for while this one is computed
-        if (handed_out && lane == 0) nb = __hip_atomic_fetch_add(&s_next[sw], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      // the row after b for this wave (handed out as waves become free, or every groups-th one)
+      auto next_of = [&](u32 b) -> u32 {
+        if (!handed_out) return b + groups;
+        u32 nb = 0u;
+        if (lane == 0) nb = __hip_atomic_fetch_add(&s_next[sw], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(nb)));
+      };
+      // One step: the wave's next row is asked for into `nxt`, then row b (in `cur`) is computed.  The next row is asked
+      // for always: when there is none it is the last row once more (from the cache, ignored) - a branch around the
+      // loads would hide from the compiler how many are in flight where it places the wait for this row's.
+      auto step = [&](typename Q::Regs (&cur)[UR], typename Q::Regs (&nxt)[UR], u32 b) -> u32 {
+        const u32 nb = next_of(b);
+        issue(nxt, slab, nb < batches ? nb : batches - 1u);
+        __builtin_amdgcn_sched_barrier(0);      // (the loads stay in front of the arithmetic whatever the register pressure)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const float p = wave_sum_lane63(Q::dot(regs[u], c, xr, sx));
+        for (int u = 0; u < UR; ++u) {
+          const float p = wave_sum_lane63(Q::dot(cur[u], c, xr, sx));
           if (lane == 63u) {
-            const u32 idx = sw * rows_per_block + b * U + u;
+            const u32 idx = sw * rows_per_block + b * UR + u;
             part[idx] = (slab == sw) ? p : part[idx] + p;
           }
         }
-        if (handed_out) {
-          b = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(nb)));
-        } else {
-          b += groups;
-        }
+        return nb;
+      };
+      u32 b = grp;
+      if (slab != sw) issue(regs, slab, b);
+      while (true) {
+        b = step(regs, regs_b, b);
+        if (b >= batches) break;
+        b = step(regs_b, regs, b);
+        if (b >= batches) break;
       }
     }
   }
