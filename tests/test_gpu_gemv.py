@@ -7,6 +7,7 @@ import pytest
 
 import trueno_amd as t
 from oracle import kquant as kq
+from trueno_amd import _ffi
 from tests.kq_helpers import REF_SLACK, gpu_gemv, record_ratio
 
 pytestmark = pytest.mark.gpu
@@ -136,3 +137,22 @@ def test_gemv_linearity_full_size(gpu):
     y2 = gpu_gemv(gpu, "q4k", buf, x2, k, n).astype(np.float64)
     y12 = gpu_gemv(gpu, "q4k", buf, (2.0 * x1 - 0.5 * x2).astype(np.float32), k, n)
     assert kq.rel_l2(y12, 2.0 * y1 - 0.5 * y2) <= 5e-6
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (32000, 4096), (515, 2048), (129, 1024), (64, 256), (1001, 4096), (2, 4096),
+                                 (4097, 3840)])
+def test_q6k_streamed_through_lds_gives_the_bits_of_the_register_form(gpu, n, k):
+    """Q6_K rows streamed through LDS (opt-in: "gemv_stream_q6k") lie there with their 210-byte blocks re-spaced to 224;
+    the arithmetic is the register form's, so every bit must be.  Weights at several alignments (a block may start at any
+    even address), ragged row counts (the last batch of a matrix starts early), short rows (fewer pieces than a slot)."""
+    tune = lambda key, v: _ffi.lib().trn_set_tuning(key.encode(), int(v))
+    buf, x = kq.gen_matrix("q6k", 100 + n, n, k), kq.gen_x(7, k)
+    for w_off in (0, 2, 6):
+        a = gpu_gemv(gpu, "q6k", buf, x, k, n, w_offset=w_off)
+        assert tune("gemv_stream_q6k", 1) == 0 and tune("gemv_stream_min_rows", 1) == 0
+        try:
+            b = gpu_gemv(gpu, "q6k", buf, x, k, n, w_offset=w_off)
+        finally:
+            tune("gemv_stream_q6k", 0)
+            tune("gemv_stream_min_rows", 0)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (n, k, w_off)

@@ -188,6 +188,26 @@ def test_many_entries_whatever_the_weights_of_the_cut(gpu, item_kb, slab_weight)
         assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), name
 
 
+def test_many_entries_with_q6k_streamed_through_lds(gpu):
+    """A large launch of one-slab matrices in workgroups of eight waves, Q6_K streamed through LDS as well (both opt-in):
+    the bits of one launch per entry."""
+    rng = np.random.default_rng(11)
+    specs = [(("q6k", "q4k", "q6k")[i % 3], int(rng.choice((2, 31, 640, 2817))), int(rng.choice((256, 1024, 4096))),
+              "x", f"y{i}", int(rng.integers(2))) for i in range(36)]
+    sep, _ = _run(gpu, specs, 4096, 1)
+    try:
+        _tune("gemv_stream_q6k", 1)
+        _tune("many_waves", 8)
+        plan = []
+        got, _ = _run(gpu, specs, 4096, 0, plan)
+    finally:
+        _tune("gemv_stream_q6k", 0)
+        _tune("many_waves", 0)
+    assert max(plan) == 0, plan
+    for name in sep:
+        assert np.array_equal(sep[name].view(np.uint32), got[name].view(np.uint32)), name
+
+
 def test_many_entries_plan_is_reused_and_replaced(gpu):
     """The cut of a list and its device tables are kept per stream for as long as the same list comes again; another list
     replaces them.  Two lists issued alternately on one stream, each twice in a row: always the bits of one launch per entry."""

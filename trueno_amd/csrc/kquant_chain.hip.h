@@ -128,16 +128,15 @@ __device__ __forceinline__ bool chain_wait(u32* barrier, u32 spin_limit, u32* st
 // from LDS (Quarter::load_lds: the same pieces as Quarter::load takes from memory).  The arithmetic - and so every bit of
 // the result - is chain_step's.
 //
-// A batch may start at any even address (Q6_K rows of 210-byte blocks): the copy starts at the 16-byte boundary below it
-// and the reads are shifted by the difference.  Pieces beyond the end of the batch (or of the matrix) repeat its last
-// piece: a batch is always the same number of wave instructions, so the number of copies outstanding is known where
-// the waits are written (vmcnt counted by hand; all LDS traffic in asm, see kquant_quarter.hip.h).
+// Q4_K and Q5_K rows are whole 16-byte pieces and lie in LDS as in memory; Q6_K blocks (210 bytes, at any even address) are
+// re-spaced to 224 bytes by the copy, see below.  Pieces beyond the end of the batch repeat its last piece: a batch is
+// always the same number of wave instructions, so the number of copies outstanding is known where the waits are written
+// (vmcnt counted by hand; all LDS traffic in asm, see kquant_quarter.hip.h).
 //   LDS: [k floats of x, swizzled][rows_per_block partial sums][64 group sums of squares][ring: waves * 2 * slot bytes]
 // ------------------------------------------------------------------------------------------------------------
 template <int FMT, int U> struct StreamSlot {
-  // wave instructions per batch: the batch's bytes from the 16-byte boundary below its first one (Q6_K rows can start
-  // at any even address) in KB
-  static constexpr u32 PIECES = (U * 16u * Quarter<FMT>::SB + (FMT == FMT_Q6K ? 15u : 0u) + 1023u) / 1024u;
+  // wave instructions per batch (64 pieces of 16 bytes each): the batch's bytes in LDS, a Q6_K block taking 224
+  static constexpr u32 PIECES = (U * 16u * (FMT == FMT_Q6K ? 224u : Quarter<FMT>::SB) + 1023u) / 1024u;
   static constexpr u32 BYTES = PIECES * 1024u;
 };
 
@@ -173,23 +172,36 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
   const u32 lds_next = lds_addr_of(&s_next_stream);
 
   // Batch b of this workgroup into ring slot `slot`; returns the byte shift of the batch inside the slot.
-  // Wave instruction j copies the 64 pieces 64 j .. 64 j + 63 of the batch; pieces behind the last byte of the batch
-  // repeat its last piece (the bytes behind a matrix need not exist), and a batch that does not exist is NL times the
-  // first piece of the matrix (one line, from the cache).  One form for every case, so that a batch is the same
-  // number of copies on every path: a branch between forms is two branches in the assembly, with a path that takes
-  // neither as far as a reader of the assembly can tell.
-  // Q4_K / Q5_K: rows are whole 16-byte pieces, so a batch starts on a piece and which piece a lane copies with which
-  // instruction is the same for every batch: the offsets are formed once (pieces behind the batch's last repeat it).  A
-  // batch that would reach behind the matrix starts as many rows early instead and its rows are found further into the
-  // slot; one that does not exist reads the matrix's first batch.
-  constexpr bool kPieceAligned = FMT != FMT_Q6K;
-  [[maybe_unused]] u32 piece_off[NL];
-  if constexpr (kPieceAligned) {
+  // Wave instruction j copies the 64 pieces 64 j .. 64 j + 63 of the batch; which bytes of the batch a lane copies with
+  // which instruction is the same for every batch, so the offsets are formed once.  Pieces behind the batch's last
+  // repeat it, and a batch that does not exist reads the matrix's first batch (from the cache).  A batch that would
+  // reach behind the matrix starts as many rows early instead and its rows are found further into the slot.  One form
+  // for every case, so that a batch is the same number of copies on every path: a branch between forms is two branches
+  // in the assembly, with a path that takes neither as far as a reader of the assembly can tell.
+  // Q6_K: a block is 210 bytes, so in a copy of the memory as it lies most blocks would sit at 2-byte alignment in LDS,
+  // and a 16-byte LDS read that is not 16-byte aligned takes eight times as long as one that is (27 against 3.4 ns per
+  // wave instruction and CU, measured).  So the copy re-spaces the blocks: a lane's 16 bytes may come from any address,
+  // and block i of a row goes to 224 i - pieces 0..12 are its bytes 0..207, piece 13 its last 16 bytes (194..209, so d
+  // is found at 222 and nothing behind the block is read).  The pieces then come from 2-byte-aligned addresses, which
+  // costs the copy (17-22 against 9 ns per wave instruction and CU) far less than it saves the reads.
+  constexpr bool kGather = FMT == FMT_Q6K;
+  constexpr u32 kPitch = kGather ? 224u : Q::SB;                     // of a block in LDS
+  const u32 row_pitch = nsb * kPitch;                                // of a row in LDS
+  u32 piece_off[NL];
+  if constexpr (!kGather) {
     const u32 last = (batch_bytes - 1u) >> 4;
 #pragma unroll
     for (u32 j = 0; j < NL; ++j) {
       const u32 p = 64u * j + lane;
       piece_off[j] = 16u * (p < last ? p : last);
+    }
+  } else {
+    const u32 per_row = 14u * nsb, pieces = U * per_row;
+#pragma unroll
+    for (u32 j = 0; j < NL; ++j) {
+      const u32 p = 64u * j + lane, pc = p < pieces ? p : pieces - 1u;
+      const u32 u = pc / per_row, r = pc - u * per_row, blk = r / 14u, jj = r - 14u * blk;
+      piece_off[j] = u * row_bytes + blk * Q::SB + (jj < 13u ? 16u * jj : Q::SB - 16u);
     }
   }
   auto issue = [&](u32 b, u32 slot) -> u32 {
@@ -197,29 +209,16 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
     const bool exists = b < batches && off < total;
     if (!exists) off = 0;
     const u32 dst = lds_ring + slot * Slot::BYTES;
-    if constexpr (kPieceAligned) {
-      u32 shift = 0;
-      if (total - off < batch_bytes) {                                // (total >= batch_bytes: the launcher streams no matrix of fewer than U rows)
-        shift = batch_bytes - static_cast<u32>(total - off);
-        off = total - batch_bytes;
-      }
-      const uint8_t* src = e.w + off;
-#pragma unroll
-      for (u32 j = 0; j < NL; ++j) dma16_nt(src + piece_off[j], dst + 1024u * j);
-      return shift;
-    } else {
-      const u32 avail = static_cast<u32>(total - off < batch_bytes ? total - off : batch_bytes);
-      const uint8_t* src = e.w + off;
-      const u32 shift = static_cast<u32>(reinterpret_cast<size_t>(src)) & 15u;
-      src -= shift;
-      const u32 last = exists ? (shift + avail - 1u) >> 4 : 0u;       // the last 16-byte piece that holds bytes of the batch
-#pragma unroll
-      for (u32 j = 0; j < NL; ++j) {
-        const u32 p = 64u * j + lane;
-        dma16_nt(src + 16u * (p < last ? p : last), dst + 1024u * j);
-      }
-      return shift;
+    u32 shift = 0;
+    if (total - off < batch_bytes) {                                  // (total >= batch_bytes: the launcher streams no matrix of fewer than U rows)
+      const u32 missing = batch_bytes - static_cast<u32>(total - off);   // whole rows
+      shift = kGather ? missing / Q::SB * kPitch : missing;
+      off = total - batch_bytes;
     }
+    const uint8_t* src = e.w + off;
+#pragma unroll
+    for (u32 j = 0; j < NL; ++j) dma16_nt(src + piece_off[j], dst + 1024u * j);
+    return shift;
   };
 
   // Activations first (loads return in order, and the vector is an L2 hit), then the first two batches of this wave.
@@ -322,10 +321,10 @@ __device__ __forceinline__ bool chain_step_stream(const ChainEntry& e, f32x4* ld
       if (nxt_in_flight) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       const u32 slot = it & 1u;
-      const u32 base = lds_ring + slot * Slot::BYTES + shift_cur + sbc * Q::SB;
+      const u32 base = lds_ring + slot * Slot::BYTES + shift_cur + sbc * kPitch;
       const u32 rows_here = n_dim - (row0 + cur * U);               // (>= 1) rows behind the matrix's last re-read it: never stored
 #pragma unroll
-      for (int u = 0; u < U; ++u) Q::load_lds(regs[u], base + (static_cast<u32>(u) < rows_here ? u : rows_here - 1u) * row_bytes, c);
+      for (int u = 0; u < U; ++u) Q::load_lds(regs[u], base + (static_cast<u32>(u) < rows_here ? u : rows_here - 1u) * row_pitch, c);
       // the batch after the next: handed out among the waves as they become free (the memory system does not serve
       // them evenly); its copies go where the current batch was, which is in registers when the reads have returned
       u32 nn;

@@ -260,13 +260,15 @@ template <> struct Quarter<FMT_Q6K> {
     r.d = load16_a2(base + off + 208);
   }
 
-  static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {       // blocks lie at 2-byte alignment in LDS too
+  // From the copy in LDS, where the block starts on a 16-byte boundary and its last 16 bytes (194..209) lie at 208: d
+  // is the half word at 222.
+  static __device__ __forceinline__ void load_lds(Regs& r, u32 blk, u32 c) {
     const u32 h = c >> 1, is = c & 1u;
     ldsq_read128<0>(r.a, blk + 64u * h + 16u * is);
     ldsq_read128<32>(r.b, blk + 64u * h + 16u * is);
     ldsq_read128<128>(r.c, blk + 32u * h + 16u * is);
     ldsq_read64<192>(r.sc, blk + 8u * h);
-    ldsq_read16<208>(r.d, blk);
+    ldsq_read16<222>(r.d, blk);
   }
   static __device__ __forceinline__ void landed(Regs& r) { asm volatile("" : "+v"(r.a), "+v"(r.b), "+v"(r.c), "+v"(r.sc), "+v"(r.d)); }
 

@@ -65,10 +65,10 @@ constexpr uint32_t kFastLdsLimit = 64 * 1024;  // dynamic LDS the fast kernels m
 constexpr uint32_t kLdsScratch = 64 + 256;     // group sums of squares (k/256 <= 64 floats) at the end of the fast kernels' LDS
 // The engine for matrices of one slab (k <= 4096) streams the rows through LDS (chain_step_stream of kquant_chain.hip.h):
 // behind the vector, the partial sums and the scratch every wave owns a ring of two slots of this many bytes (a batch of
-// KQ_U rows of 16 blocks, from the 16-byte boundary below its first byte, in whole KB: StreamSlot of the kernels).
+// KQ_U rows of 16 blocks as they lie in LDS - a Q6_K block takes 224 bytes there - in whole KB: StreamSlot of the kernels).
 constexpr uint32_t kChainStreamFlag = 16u;     // CHAIN_STREAM_LDS
 constexpr uint32_t kStreamLdsLimit = 160 * 1024 - 1024;   // dynamic LDS such a launch may ask for (the CU has 160 KB; static LDS is a few words)
-constexpr uint32_t stream_slot_bytes(uint32_t sb_bytes) { return (kGemvRowsPerBatch * 16u * sb_bytes + (sb_bytes == 210u ? 15u : 0u) + 1023u) / 1024u * 1024u; }
+constexpr uint32_t stream_slot_bytes(uint32_t sb_bytes) { return (kGemvRowsPerBatch * 16u * (sb_bytes == 210u ? 224u : sb_bytes) + 1023u) / 1024u * 1024u; }
 
 struct DeviceKernels {
   bool loaded = false;
@@ -222,9 +222,10 @@ struct GemvGeometry {
 };
 
 // Can an n x k matrix of this format go through the streamed engine?  (one slab; any alignment the fast kernels take)
-// Q6_K stays on the register path: its 210-byte blocks lie at 2-byte alignment in LDS too, and the five reads per row
-// that start there cost more than the whole-line copies gain (eight 4096 x 4096 per call 3.18 -> 3.38 us a matrix,
-// 32000 x 4096 19.4 -> 19.9 us; Q4_K 11008 x 4096 5.02 -> 4.53 us, Q5_K 6.57 -> 6.29 us).  "gemv_stream_q6k" turns it on.
+// Q6_K stays on the register path by default: its slots are 7 KB (the 210-byte blocks re-spaced to 224), so a workgroup
+// of twelve waves has no room for its rings, and a launch alone gains nothing (32000 x 4096: 19.2-20 us either way).  A
+// long list of one-slab Q6_K matrices in workgroups of eight waves ("many_waves") is 4-7 % faster streamed (64 matrices
+// of 4096 x 4096: 144 against 155 us; eight of 32000 x 4096: 138 against 147 us).  "gemv_stream_q6k" turns it on.
 bool stream_ok(uint32_t fmt_code, uint32_t k, uint32_t n) {
   return !g_tune_stream_off && k != 0 && k <= 4096u && n >= kGemvRowsPerBatch && (fmt_code != 6u || g_tune_stream_q6k);
 }
