@@ -317,14 +317,14 @@ TRN_API trn_status trn_device_cu_count(int* count);
  * looks for entries (0 = twice group_max); "group_waves": least waves per workgroup of a launch of up to sixteen entries (0 = 8,
  * or what its widest entry needs); "many_waves": waves per workgroup of a launch of more than sixteen entries (0 = 12);
  * "group_slab_weight": percent added to an entry's bytes per further 4096 columns when a launch of up to sixteen entries
- * shares out its workgroups (0 = 40); "many_slab_weight": the same for a launch of more than sixteen (0 = 18);
+ * shares out its workgroups (0 = 40); "many_slab_weight": the same for a launch of more than sixteen (0 = 13);
  * "many_item_kb": what every piece of an entry costs the workgroup that takes it, in KB of weights (0 = 64).
  * "gemv_stream_off": 1 = no matrix streams its rows through LDS (every GEMV loads its rows into registers straight from
  * memory; same bits); "gemv_stream_q6k": 1 = Q6_K matrices of up to 4096 columns stream too (their slots are larger:
  * in a launch of more than sixteen entries only with "many_waves" of 10 or less; 4-7 % faster on long lists at 8);
  * "gemv_stream_waves": waves per workgroup of a single streamed GEMV (0 = 4); "gemv_stream_min_rows": a single GEMV
  * streams when a wave gets at least this many rows (0 = 16); "group_stream_min_rows": the same for an entry of a launch
- * of up to sixteen entries (0 = 16); "gemv_stream_cost": percent of its bytes a streamed entry
+ * of up to sixteen entries (0 = 24); "gemv_stream_cost": percent of its bytes a streamed entry
  * counts for when a launch shares out its workgroups (0 = 95).
  * "gemm_few": the Q4_K product of two to four tokens on the integer matrix cores - 0 = where its estimated time is the
  * lowest, 1 = wherever it can run, 2 = never.

@@ -771,13 +771,16 @@ constexpr double kSlabCost = 0.4;
 // what a streamed entry's bytes cost against an entry's on the register path (launch_gemv_group)
 constexpr double kStreamCost = 0.95;
 // rows a wave must get for an entry of a launch of up to sixteen to stream: the strict decoder chain 1370 / 1381 / 1356 / 1338 / 1336 /
-// 1334 us with 1 / 4 / 8 / 12 / 16 / 24 (its launches of one to three entries leave a wave 6-11 rows); the pass with shared buffers within its scatter
-constexpr double kGroupStreamMinRows = 16.0;
+// 1334 us with 1 / 4 / 8 / 12 / 16 / 24 (its launches of one to three entries leave a wave 6-11 rows).  Since the register form
+// asks for a wave's next row while it computes this one, the pass with shared buffers (65 launches) takes 1030 / 999 / 998 /
+// 999 us with 16 / 24 / 48 / never; the strict chain does not care (1270 us).
+constexpr double kGroupStreamMinRows = 24.0;
 // launches of more than sixteen entries (plan_gemv_many): weight per further slab and what a piece of work costs a workgroup
 // (KB of weights).  The 7B pass: 730 / 718 / 704 / 702 / 702 / 708 / 711 us with 40 / 30 / 25 / 20 / 15 / 10 / 5 % per slab (with 40 %
 // the workgroups with the one-slab o matrices ended 35 us after those with the three-slab down matrices); the cost of a piece
-// made no difference between 1 and 128 KB, more was slower.
-constexpr double kManySlabCost = 0.18, kManyItemKb = 64.0;
+// made no difference between 1 and 128 KB, more was slower.  With the register form's rows double-buffered and its loads
+// global (the three-slab rows 8 % faster): 672 / 664 / 661 / 659 / 660 / 678 / 688 us with 18 / 16 / 14 / 13 / 10 / 22 / 26 %.
+constexpr double kManySlabCost = 0.13, kManyItemKb = 64.0;
 // Entries a launch takes by default: as many as the kernel holds, looked for among the next 32 of the list.  On the 7B
 // pass with activation buffers per layer: 8 entries (138 MB a launch, 30 launches) 879 us, 12 of the next 24 (21
 // launches) 820 us, 14 of 28 (18) 821 us, 16 of 32 (16 launches of 270 MB) 823 us; the launches of 12-16 entries run at
